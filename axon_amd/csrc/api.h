@@ -202,6 +202,15 @@ int axk_embed_scaled(const int32_t* tokens, const void* table, int packed, float
 // (elem [n_rows, dim], or null) also gets the new x in the compute dtype.
 int axk_norm_add(const float* y, const void* gain, int gain_is_f32, float eps, float mult, float* x, void* rounded,
                  int n_rows, int dim, void* stream);
+// x[r, :] = norm(alpha x[r, :] + y[r, :]) * gain: the norm behind the sum; kind 0: an RMS norm, kind 1: a
+// layer norm (mean taken off, the variance the mean of the squared deviations).  `rounded` as above.
+int axk_sum_norm(const float* y, float alpha, const void* gain, int gain_is_f32, float eps, int kind, float* x, void* rounded,
+                 int n_rows, int dim, void* stream);
+// Layer norm with a gain and no bias of float32 rows (rows: which, or null for all) into the compute dtype.
+int axk_layernorm(const float* x, const int32_t* rows, const void* gain, int gain_is_f32, void* out, int n_rows, int dim,
+                  float eps, void* stream);
+// v[r, i] = cap tanh(v[r, i] / cap), in place on float32 rows row_stride apart.
+int axk_softcap(float* v, long row_stride, int n_rows, int n, float cap, void* stream);
 // out[i] = x[i] in the compute dtype.
 int axk_round_rows(const float* x, void* out, long n, void* stream);
 // out[t, :] = [a[t, :] | b[t, :]] in the compute dtype (a [n_rows, wa], b [n_rows, wb] float32).
@@ -219,18 +228,24 @@ int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, flo
 // tile_rows 16, or 64 for many rows a group: tiles through LDS, the same chains, the same bits): the rows
 // listed, x_rows / out_rows naming the row of X each reads and the row of out it writes (null:
 // the listed row itself).  glu: g = min(gate, limit), u = clamp(up, -limit, limit), out = g
-// sigmoid(alpha g) (u + 1).  gate (float32, rows gate_row_stride apart): out is multiplied by
-// sigmoid(gate[orow, g ogs + n]).  Strides count elements.  An output's chain over k depends on
+// sigmoid(alpha g) (u + shift); an infinite limit, alpha 1 and shift 0 are silu(gate) up.  gate (float32,
+// rows gate_row_stride apart): out is multiplied by sigmoid(gate[orow, g ogs + n]), or with
+// gate_per_group by sigmoid(gate[orow, g]), one number a group.  Strides count elements.  An output's chain over k depends on
 // k, the strides' alignment and the build alone (axk_grouped_gemm_uses_mfma says which chain).
 int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride, long x_group_stride);
 int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
                      const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32, long out_row_stride,
-                     long out_group_stride, const int32_t* out_rows, const float* gate, long gate_row_stride, int glu,
-                     float glu_limit, float glu_alpha, const int32_t* tiles, const int32_t* n_tiles, int max_tiles,
+                     long out_group_stride, const int32_t* out_rows, const float* gate, long gate_row_stride,
+                     int gate_per_group, int glu, float glu_limit, float glu_alpha, float glu_shift, const int32_t* tiles,
+                     const int32_t* n_tiles, int max_tiles,
                      int tile_rows, int m, int n, int k, int groups, void* stream);
 
 // Routing (csrc/moe.hip).  axk_route_topk: for each token the `top` largest of its n_experts
 // logits (the largest first; of equal ones the lower expert) and the softmax over these.
+// axk_route_scored: scores s = sigmoid(logits) that do not compete; chosen by s + correction (float32
+// [n_experts], or null) among the experts of the `keep` best of `groups` equal groups of neighbours (a
+// group's score: the sum of its two largest choice scores), weights s / (sum of the chosen s + 1e-20)
+// * scale.  Up to 1,024 experts in up to 64 groups, up to 64 a token.
 // axk_route_sort: the pairs p = t top + k in expert order (sorted, and each one's token in
 // sorted_tokens) and the tiles (of up to tile_rows rows) of the grouped product, at most
 // axk_route_max_tiles of them.
@@ -239,6 +254,8 @@ int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_grou
 // axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending (with
 // place_of: rows[place_of[t top + k], :]).  axk_gather_rows: out[r, :] = x[rows[r], :] (elem).
 int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights, void* stream);
+int axk_route_scored(const float* logits, const float* correction, int n_tokens, int n_experts, int top, int groups, int keep,
+                     float scale, int32_t* experts, float* weights, void* stream);
 int axk_route_max_tiles(int n_pairs, int n_experts, int tile_rows);
 int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted, int32_t* sorted_tokens,
                    int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of, int tile_rows, void* stream);
@@ -275,22 +292,26 @@ int axk_gated_scan(const float* gates, const float* u, const void* y, long y_str
 // axk_latent_prepare: from the float32 rows of the down projections, the normed query latent
 // (cq elem [T, q_rank]; q_rank 0: none) and, with write_kv, the normed key/value latent and the
 // rotated shared key part into the request's page.  axk_latent_query_rope: the rotated part of
-// every head's query into q_full [T, heads, rank + rot] (places rank ..).  axk_latent_attention:
-// o_lat [T, heads, rank] = softmax over lo ..= pos of (q_full . page row) scale, times the rows'
-// first `rank` places; lo = window > 0 ? max(0, pos + 1 - window) : 0.
+// every head's query (q float32, rows q_stride apart) into q_full [T, heads, rank + rot] (places rank ..).
+// Rotation: pairs (i, i + rot_dims / 2), or (2i, 2i + 1) with `neighbours`; cos and sin times `magnitude`.
+// axk_latent_attention: o_lat [T, heads, rank] = softmax over lo ..= pos of (q_full . page row) scale, times
+// the rows' first `rank` places; lo = window > 0 ? max(0, pos + 1 - window) : 0.  sink (float32 [heads], or
+// null): the softmax's denominator also holds exp(sink[head]), once, with no value.
 int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, int kv_at, int rank, int rot, int rot_dims,
-                       const void* q_gain, int q_gain_is_f32, const void* kv_gain, int kv_gain_is_f32, float eps,
+                       int neighbours, float magnitude, const void* q_gain, int q_gain_is_f32, const void* kv_gain, int kv_gain_is_f32, float eps,
                        const float* table, const int32_t* positions, const int32_t* seq_rows, const int32_t* block_table,
                        int table_stride, void* cache, int page_size, void* cq, int n_tokens, int write_kv, void* stream);
-int axk_latent_query_rope(const float* q, int dim, int rot, int rot_dims, const float* table, float* q_full, int rank,
-                          int heads, int n_tokens, void* stream);
-// partial: axk_latent_attention_workspace floats (0 for most calls; with few tokens over a window the
-// blocks of 64 positions of a token then run side by side and a second launch folds them), or null.
+int axk_latent_query_rope(const float* q, long q_stride, int dim, int rot, int rot_dims, int neighbours, float magnitude,
+                          const float* table, float* q_full, int rank, int heads, int n_tokens, void* stream);
+// partial: axk_latent_attention_workspace floats (0 for most calls; with few tokens the blocks of 64
+// positions of a token then run side by side and a second launch folds them), or null.  span: the most
+// positions a row of the step sees, for attention without a window (0: not known).
 int axk_latent_attention_uses_mfma(int heads, int rank, int rot, int page_size);
-long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window);
+long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window, int span);
 int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                          const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
-                         int rot, int page_size, int window, float scale, float* partial, long partial_floats, void* stream);
+                         int rot, int page_size, int window, int span, float scale, const float* sink, float* partial,
+                         long partial_floats, void* stream);
 
 // Grouped-query attention with one or two score maps a head, an optional norm of queries and keys, a
 // sliding-window or chunked mask, bent scores and a gate (csrc/masked_attention.hip).  A page is

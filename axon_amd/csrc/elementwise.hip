@@ -285,6 +285,120 @@ extern "C" int axk_norm_add(const float* y, const void* gain, int gain_is_f32, f
   return 0;
 }
 
+// ---------------------------------------------------------------------------- layer norm (a gain, no bias)
+// mean = sum x / n, var = sum (x - mean)^2 / n (a second pass over the deviations, not E[x^2] - mean^2),
+// out = ((x - mean) * 1 / sqrt(var + eps)) * g.  Both sums as in rmsnorm_kernel: a strided chain per
+// thread, a butterfly per wave, the four waves in order.
+__global__ void __launch_bounds__(NORM_THREADS)
+layernorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows, const void* __restrict__ gain,
+                 int gain_is_f32, elem_t* __restrict__ out, int dim, float eps) {
+  __shared__ float partial[2][NORM_THREADS / AXON_WAVE];
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * dim;
+  float sum = 0.0f;
+  for (int i = threadIdx.x; i < dim; i += NORM_THREADS) sum += src[i];
+  const float mean = block_sum_256(sum, partial[0]) / (float)dim;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < dim; i += NORM_THREADS) {
+    const float d = src[i] - mean;
+    ss = fmaf(d, d, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, partial[1]) / (float)dim + eps);
+  elem_t* dst = out + (size_t)r * dim;
+  for (int i = threadIdx.x; i < dim; i += NORM_THREADS)
+    dst[i] = from_float(((src[i] - mean) * inv) * load_vec(gain, gain_is_f32, i));
+}
+
+extern "C" int axk_layernorm(const float* x, const int32_t* rows, const void* gain, int gain_is_f32, void* out, int n_rows,
+                             int dim, float eps, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && dim > 0, "layernorm: bad sizes rows=%d dim=%d", n_rows, dim);
+  if (n_rows == 0) return 0;
+  layernorm_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim, eps);
+  AXK_LAUNCH_CHECK("layernorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- a norm behind the sum
+// x[r, :] = norm(alpha x[r, :] + y[r, :]) * gain, the norm an RMS norm (kind 0) or a layer norm (kind 1,
+// as layernorm_kernel), and rounded[r, :] = the new x[r, :] in the compute dtype if asked for (what the
+// next sublayer's products read).  A thread keeps its first POST_KEPT sums in registers (rows up to
+// 4,096 wide are read once); beyond that it adds them again.
+#define POST_KEPT 16
+__global__ void __launch_bounds__(NORM_THREADS)
+sum_norm_kernel(const float* __restrict__ y, float alpha, const void* __restrict__ gain, int gain_is_f32, float eps, int kind,
+                float* __restrict__ x, elem_t* __restrict__ rounded, int dim) {
+  __shared__ float partial[2][NORM_THREADS / AXON_WAVE];
+  const int r = blockIdx.x;
+  const float* add = y + (size_t)r * dim;
+  float* row = x + (size_t)r * dim;
+  float kept[POST_KEPT];
+#pragma unroll
+  for (int c = 0; c < POST_KEPT; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    kept[c] = i < dim ? alpha * row[i] + add[i] : 0.0f;
+  }
+  float mean = 0.0f;
+  if (kind == 1) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < POST_KEPT; ++c) sum += kept[c];
+    for (int i = threadIdx.x + POST_KEPT * NORM_THREADS; i < dim; i += NORM_THREADS) sum += alpha * row[i] + add[i];
+    mean = block_sum_256(sum, partial[0]) / (float)dim;
+  }
+  float ss = 0.0f;
+#pragma unroll
+  for (int c = 0; c < POST_KEPT; ++c) {
+    const float d = threadIdx.x + c * NORM_THREADS < dim ? kept[c] - mean : 0.0f;
+    ss = fmaf(d, d, ss);
+  }
+  for (int i = threadIdx.x + POST_KEPT * NORM_THREADS; i < dim; i += NORM_THREADS) {
+    const float d = (alpha * row[i] + add[i]) - mean;
+    ss = fmaf(d, d, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, partial[1]) / (float)dim + eps);
+#pragma unroll
+  for (int c = 0; c < POST_KEPT; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    if (i < dim) {
+      const float v = ((kept[c] - mean) * inv) * load_vec(gain, gain_is_f32, i);
+      row[i] = v;
+      if (rounded) rounded[(size_t)r * dim + i] = from_float(v);
+    }
+  }
+  for (int i = threadIdx.x + POST_KEPT * NORM_THREADS; i < dim; i += NORM_THREADS) {
+    const float v = (((alpha * row[i] + add[i]) - mean) * inv) * load_vec(gain, gain_is_f32, i);
+    row[i] = v;
+    if (rounded) rounded[(size_t)r * dim + i] = from_float(v);
+  }
+}
+
+extern "C" int axk_sum_norm(const float* y, float alpha, const void* gain, int gain_is_f32, float eps, int kind, float* x,
+                            void* rounded, int n_rows, int dim, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && dim > 0 && (kind == 0 || kind == 1), "sum_norm: bad sizes rows=%d dim=%d kind=%d", n_rows, dim, kind);
+  if (n_rows == 0) return 0;
+  sum_norm_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(y, alpha, gain, gain_is_f32, eps, kind, x, (elem_t*)rounded, dim);
+  AXK_LAUNCH_CHECK("sum_norm");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- bent logits
+// v[r, i] = cap tanh(v[r, i] / cap), in place on float32 rows.
+__global__ void softcap_kernel(float* __restrict__ v, long row_stride, int n, float cap) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    float* at = v + (long)blockIdx.y * row_stride + i;
+    *at = cap * tanhf(*at / cap);
+  }
+}
+
+extern "C" int axk_softcap(float* v, long row_stride, int n_rows, int n, float cap, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n_rows <= 65535 && n > 0 && cap > 0.0f, "softcap: bad sizes rows=%d n=%d cap=%g", n_rows, n, (double)cap);
+  if (n_rows == 0) return 0;
+  softcap_kernel<<<dim3(ceil_div(n, 256), n_rows), 256, 0, (hipStream_t)stream>>>(v, row_stride, n, cap);
+  AXK_LAUNCH_CHECK("softcap");
+  return 0;
+}
+
 // out[i] = x[i] in the compute dtype.
 __global__ void round_rows_kernel(const float* __restrict__ x, elem_t* __restrict__ out, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -12,8 +12,9 @@
 //     The grid is launched for the most tiles there can be; blocks beyond *n_tiles leave at once.
 //
 // Epilogues: bias; a gated linear unit with clamps (W holds 2 N rows a group, gate rows then up
-// rows: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + 1));
-// a multiplication by sigmoid(gate[orow, g ogs + n]); out in float32 or in the compute dtype.
+// rows: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + shift); an
+// infinite limit, alpha 1 and shift 0 give silu(gate) up); a multiplication by sigmoid(gate[orow, g ogs + n]),
+// or by sigmoid(gate[orow, g]), one number a group; out in float32 or in the compute dtype.
 //
 // The K-reduction of one output is one chain in ascending k that depends on K and the build alone
 // (32-bit FMA, or 16x16x32 MFMAs where the bfloat16 build can use them: K a multiple of 32 and
@@ -28,8 +29,8 @@ struct GroupedArgs {
   const void* x; int x_is_f32; long x_row_stride; long x_group_stride; const int32_t* x_rows;
   const elem_t* w; const void* bias; int bias_is_f32;
   void* out; int out_is_f32; long out_row_stride; long out_group_stride; const int32_t* out_rows;
-  const float* gate; long gate_row_stride;
-  int glu; float glu_limit; float glu_alpha;
+  const float* gate; long gate_row_stride; int gate_per_group;
+  int glu; float glu_limit; float glu_alpha; float glu_shift;
   const int32_t* tiles; const int32_t* n_tiles;
   int M, N, K, G;
 };
@@ -42,10 +43,10 @@ __device__ inline float gg_load_x(const GroupedArgs& a, long at) {
   return a.x_is_f32 ? ((const float*)a.x)[at] : to_float(((const elem_t*)a.x)[at]);
 }
 
-__device__ inline float clamped_glu(float gate, float up, float limit, float alpha) {
+__device__ inline float clamped_glu(float gate, float up, float limit, float alpha, float shift) {
   const float g = fminf(gate, limit);
   const float u = fminf(fmaxf(up, -limit), limit);
-  return (g * (1.0f / (1.0f + expf(-(alpha * g))))) * (u + 1.0f);
+  return (g * (1.0f / (1.0f + expf(-(alpha * g))))) * (u + shift);
 }
 
 __device__ inline void gg_store(const GroupedArgs& a, int g, int orow, int n, float v, float up) {
@@ -54,9 +55,9 @@ __device__ inline void gg_store(const GroupedArgs& a, int g, int orow, int n, fl
     v += load_vec(a.bias, a.bias_is_f32, g * per + n);
     if (a.glu) up += load_vec(a.bias, a.bias_is_f32, g * per + a.N + n);
   }
-  if (a.glu) v = clamped_glu(v, up, a.glu_limit, a.glu_alpha);
+  if (a.glu) v = clamped_glu(v, up, a.glu_limit, a.glu_alpha, a.glu_shift);
   const long col = (long)g * a.out_group_stride + n;
-  if (a.gate) v = v * (1.0f / (1.0f + expf(-a.gate[(long)orow * a.gate_row_stride + col])));
+  if (a.gate) v = v * (1.0f / (1.0f + expf(-a.gate[(long)orow * a.gate_row_stride + (a.gate_per_group ? g : col)])));
   const long at = (long)orow * a.out_row_stride + col;
   if (a.out_is_f32) ((float*)a.out)[at] = v;
   else ((elem_t*)a.out)[at] = from_float(v);
@@ -313,7 +314,8 @@ extern "C" int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride
 extern "C" int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
                                 const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32,
                                 long out_row_stride, long out_group_stride, const int32_t* out_rows, const float* gate,
-                                long gate_row_stride, int glu, float glu_limit, float glu_alpha, const int32_t* tiles,
+                                long gate_row_stride, int gate_per_group, int glu, float glu_limit, float glu_alpha,
+                                float glu_shift, const int32_t* tiles,
                                 const int32_t* n_tiles, int max_tiles, int tile_rows, int m, int n, int k, int groups,
                                 void* stream) {
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0 && groups > 0, "grouped_gemm: bad sizes M=%d N=%d K=%d groups=%d", m, n, k, groups);
@@ -326,7 +328,8 @@ extern "C" int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, 
   if (row_tiles == 0) return 0;
   AXK_REQUIRE(groups <= 65535 && ceil_div(n, GG_COLS) <= 65535, "grouped_gemm: %d groups of %d columns are too many", groups, n);
   GroupedArgs a{x, x_is_f32, x_row_stride, x_group_stride, x_rows, (const elem_t*)w, bias, bias_is_f32, out, out_is_f32,
-                out_row_stride, out_group_stride, out_rows, gate, gate_row_stride, glu, glu_limit, glu_alpha, tiles, n_tiles,
+                out_row_stride, out_group_stride, out_rows, gate, gate_row_stride, gate_per_group, glu, glu_limit, glu_alpha, glu_shift,
+                tiles, n_tiles,
                 m, n, k, groups};
   dim3 grid(row_tiles, ceil_div(n, GG_COLS), tiles ? 1 : groups);
   hipStream_t s = (hipStream_t)stream;

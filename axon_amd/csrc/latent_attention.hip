@@ -16,12 +16,13 @@ namespace {
 // One block per token.  fused [T, stride] float32 holds the down projections' results:
 //   [q_at, q_at + q_rank): the query latent -> RMS norm with q_gain -> cq [T, q_rank] (compute dtype);
 //   [kv_at, kv_at + rank): the key/value latent -> RMS norm with kv_gain -> the page;
-//   [kv_at + rank, + rot): the shared key part -> rotate-half on its first rot_dims dims -> the page.
+//   [kv_at + rank, + rot): the shared key part -> its first rot_dims dims rotated -> the page; the pairs are
+//   (i, i + rot_dims / 2), or (2i, 2i + 1) with `neighbours`, and cos and sin are multiplied by `magnitude`.
 // The sums of squares: a strided chain per thread, a butterfly per wave, the four waves in order.
 __global__ void __launch_bounds__(256)
 latent_prepare_kernel(const float* __restrict__ fused, long stride, int q_at, int q_rank, int kv_at, int rank, int rot,
-                      int rot_dims, const void* __restrict__ q_gain, int q_gain_is_f32, const void* __restrict__ kv_gain,
-                      int kv_gain_is_f32, float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
+                      int rot_dims, int neighbours, float magnitude, const void* __restrict__ q_gain, int q_gain_is_f32,
+                      const void* __restrict__ kv_gain, int kv_gain_is_f32, float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
                       const int32_t* __restrict__ seq_rows, const int32_t* __restrict__ block_table, int table_stride,
                       elem_t* __restrict__ cache, int page_size, elem_t* __restrict__ cq, int write_kv) {
   __shared__ float partial[4];
@@ -53,28 +54,35 @@ latent_prepare_kernel(const float* __restrict__ fused, long stride, int q_at, in
   const int half = rot_dims / 2;
   const float* tab = table + (long)t * half * 2;
   for (int i = threadIdx.x; i < half; i += 256) {
-    const float s = tab[2 * i], c = tab[2 * i + 1];
-    const float a = kr[i], b = kr[i + half];
-    dst[rank + i] = from_float(__fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s)));
-    dst[rank + i + half] = from_float(__fadd_rn(__fmul_rn(b, c), __fmul_rn(a, s)));
+    const float s = tab[2 * i] * magnitude, c = tab[2 * i + 1] * magnitude;
+    const int ia = neighbours ? 2 * i : i, ib = neighbours ? 2 * i + 1 : i + half;
+    const float a = kr[ia], b = kr[ib];
+    dst[rank + ia] = from_float(__fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s)));
+    dst[rank + ib] = from_float(__fadd_rn(__fmul_rn(b, c), __fmul_rn(a, s)));
   }
   for (int i = rot_dims + threadIdx.x; i < rot; i += 256) dst[rank + i] = from_float(kr[i]);
 }
 
-// The rotated part of every head's query: q [T, heads, dim + rot] float32 -> q_full [T, heads,
-// rank + rot] float32, places rank .. rank + rot - 1 (the first `rank` are the per-head product's).
-__global__ void latent_query_rope_kernel(const float* __restrict__ q, int dim, int rot, int rot_dims,
-                                         const float* __restrict__ table, float* __restrict__ q_full, int rank, int heads) {
+// The rotated part of every head's query: q [T, heads, dim + rot] float32 (rows q_stride apart) -> q_full
+// [T, heads, rank + rot] float32, places rank .. rank + rot - 1 (the first `rank` are the per-head
+// product's).  Pairs and magnitude as in latent_prepare_kernel.
+__global__ void latent_query_rope_kernel(const float* __restrict__ q, long q_stride, int dim, int rot, int rot_dims, int neighbours,
+                                         float magnitude, const float* __restrict__ table, float* __restrict__ q_full, int rank,
+                                         int heads) {
   const int t = blockIdx.x;
   const int half = rot_dims / 2;
   const float* tab = table + (long)t * half * 2;
   for (int idx = threadIdx.x; idx < heads * rot; idx += blockDim.x) {
     const int h = idx / rot, i = idx % rot;
-    const float* src = q + ((long)t * heads + h) * (dim + rot) + dim;
-    float v;
-    if (i < half) v = __fsub_rn(__fmul_rn(src[i], tab[2 * i + 1]), __fmul_rn(src[i + half], tab[2 * i]));
-    else if (i < rot_dims) v = __fadd_rn(__fmul_rn(src[i], tab[2 * (i - half) + 1]), __fmul_rn(src[i - half], tab[2 * (i - half)]));
-    else v = src[i];
+    const float* src = q + (long)t * q_stride + (long)h * (dim + rot) + dim;
+    float v = src[i];
+    if (i < rot_dims) {
+      const bool first = neighbours ? !(i & 1) : i < half;
+      const int pair = neighbours ? i >> 1 : (first ? i : i - half);
+      const int other = neighbours ? i ^ 1 : (first ? i + half : i - half);
+      const float s = tab[2 * pair] * magnitude, c = tab[2 * pair + 1] * magnitude;
+      v = first ? __fsub_rn(__fmul_rn(src[i], c), __fmul_rn(src[other], s)) : __fadd_rn(__fmul_rn(src[i], c), __fmul_rn(src[other], s));
+    }
     q_full[((long)t * heads + h) * (rank + rot) + rank + i] = v;
   }
 }
@@ -83,13 +91,15 @@ __global__ void latent_query_rope_kernel(const float* __restrict__ q, int dim, i
 // to absolute position, ascending; in a block lane j scores position 64 b + j (walking its key
 // row against the query in LDS), the block's maximum and sum are butterflies, and the running
 // (m, l, o) are rescaled block by block.  For the values lane d owns the latent dims d, d + 64, ...
-// and walks the block's positions, taking each weight from its lane.
+// and walks the block's positions, taking each weight from its lane.  `sink` (a number a head, or null):
+// the sum of the weights also holds exp(sink) once, which has no key and no value: the running
+// (m, l) start at (sink, 1).
 #define LA_WAVES 4
 __global__ void __launch_bounds__(LA_WAVES * 64)
 latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restrict__ cache,
                         const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
                         const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
-                        int rot, int page_size, int window, float scale) {
+                        int rot, int page_size, int window, float scale, const float* __restrict__ sink) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int width = rank + rot;
@@ -110,7 +120,7 @@ latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restri
   float acc[MAX_OWN];
 #pragma unroll
   for (int i = 0; i < MAX_OWN; ++i) acc[i] = 0.0f;
-  float m = -INFINITY, l = 0.0f;
+  float m = sink ? sink[h] : -INFINITY, l = sink ? 1.0f : 0.0f;
   for (int b = lo / 64; b <= pos / 64; ++b) {
     const int p = b * 64 + lane;
     const bool seen = p >= lo && p <= pos;
@@ -169,7 +179,8 @@ __global__ void __launch_bounds__(LAM_WAVES * 64)
 latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
                              const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
-                             int rot, int page_size, int window, float scale, float* __restrict__ partial, int n_chunks) {
+                             int rot, int page_size, int window, float scale, const float* __restrict__ sink,
+                             float* __restrict__ partial, int n_chunks) {
   // the sixteen heads' queries as bfloat16 in LDS, rows 16 bytes longer than their chunks so that the
   // sixteen rows a product's operand is read from fall into different banks
   constexpr int QROW = QC * 32 + 8;
@@ -202,7 +213,9 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
   la_f32x4 acc[RT];
 #pragma unroll
   for (int i = 0; i < RT; ++i) acc[i] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  float m = -INFINITY, l = 0.0f;
+  // a sink is counted once a row: here when the wave walks all blocks, else by the kernel that folds them
+  const bool sunk = sink != nullptr && partial == nullptr;
+  float m = sunk ? sink[hg * 16 + j] : -INFINITY, l = sunk ? 1.0f : 0.0f;
   // with `partial`: this wave takes one block of 64 positions (blockIdx.y after the token's first) and
   // leaves (o, m, l) unscaled for the kernel that folds a token's blocks in ascending order
   const int b_first = partial ? lo / 64 + (int)blockIdx.y : lo / 64;
@@ -307,18 +320,20 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
 
 // o_lat[row, :] = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) l_c over a row's blocks in ascending order
 // (M the largest m_c; a block that saw nothing has l = 0 and weighs nothing).  One block per (token,
-// head): the blocks' weights once into LDS, then a thread a dim.
+// head): the blocks' weights once into LDS, then a thread a dim.  With a sink, M is at least the head's
+// sink and the sum of the weights holds exp(sink - M) as well.
 __global__ void __launch_bounds__(128)
-latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks) {
+latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks,
+                             const float* __restrict__ sink, int heads) {
   extern __shared__ float weight[];
   const float* src = partial + (long)blockIdx.x * n_chunks * (rank + 2);
-  float M = -INFINITY;
+  float M = sink ? sink[blockIdx.x % heads] : -INFINITY;
   for (int c = 0; c < n_chunks; ++c)
     if (src[(long)c * (rank + 2) + rank + 1] > 0.0f) M = fmaxf(M, src[(long)c * (rank + 2) + rank]);
   for (int c = threadIdx.x; c < n_chunks; c += blockDim.x)
     weight[c] = src[(long)c * (rank + 2) + rank + 1] > 0.0f ? expf(src[(long)c * (rank + 2) + rank] - M) : 0.0f;
   __syncthreads();
-  float L = 0.0f;
+  float L = sink ? expf(sink[blockIdx.x % heads] - M) : 0.0f;
   for (int c = 0; c < n_chunks; ++c) L = fmaf(weight[c], src[(long)c * (rank + 2) + rank + 1], L);
   const float inv = 1.0f / L;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
@@ -331,13 +346,15 @@ latent_attention_fold_kernel(const float* __restrict__ partial, float* __restric
 template <int RT, int QC>
 static void launch_latent_mfma(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                                const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
-                               int rot, int page_size, int window, float scale, float* partial, int n_chunks, hipStream_t stream) {
+                               int rot, int page_size, int window, float scale, const float* sink, float* partial, int n_chunks,
+                               hipStream_t stream) {
   const long items = (long)n_tokens * (heads / 16);
   dim3 grid((unsigned)((items + LAM_WAVES - 1) / LAM_WAVES), partial ? n_chunks : 1);
   latent_attention_mfma_kernel<RT, QC><<<grid, LAM_WAVES * 64, 0, stream>>>(
       q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
-      window, scale, partial, n_chunks);
-  if (partial) latent_attention_fold_kernel<<<n_tokens * heads, 128, n_chunks * sizeof(float), stream>>>(partial, o_lat, rank, n_chunks);
+      window, scale, sink, partial, n_chunks);
+  if (partial)
+    latent_attention_fold_kernel<<<n_tokens * heads, 128, n_chunks * sizeof(float), stream>>>(partial, o_lat, rank, n_chunks, sink, heads);
 }
 #endif
 
@@ -354,7 +371,7 @@ extern "C" int axk_latent_attention_uses_mfma(int heads, int rank, int rot, int 
 }
 
 extern "C" int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, int kv_at, int rank, int rot,
-                                  int rot_dims, const void* q_gain, int q_gain_is_f32, const void* kv_gain,
+                                  int rot_dims, int neighbours, float magnitude, const void* q_gain, int q_gain_is_f32, const void* kv_gain,
                                   int kv_gain_is_f32, float eps, const float* table, const int32_t* positions,
                                   const int32_t* seq_rows, const int32_t* block_table, int table_stride, void* cache,
                                   int page_size, void* cq, int n_tokens, int write_kv, void* stream) {
@@ -365,37 +382,46 @@ extern "C" int axk_latent_prepare(const float* fused, long stride, int q_at, int
               "latent_prepare: the parts do not fit rows of %ld", stride);
   if (n_tokens == 0) return 0;
   latent_prepare_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(fused, stride, q_at, q_rank, kv_at, rank, rot, rot_dims,
-      q_gain, q_gain_is_f32, kv_gain, kv_gain_is_f32, eps, table, positions, seq_rows, block_table, table_stride,
+      neighbours, magnitude, q_gain, q_gain_is_f32, kv_gain, kv_gain_is_f32, eps, table, positions, seq_rows, block_table, table_stride,
       (elem_t*)cache, page_size, (elem_t*)cq, write_kv);
   AXK_LAUNCH_CHECK("latent_prepare");
   return 0;
 }
 
-extern "C" int axk_latent_query_rope(const float* q, int dim, int rot, int rot_dims, const float* table, float* q_full, int rank,
-                                     int heads, int n_tokens, void* stream) {
+extern "C" int axk_latent_query_rope(const float* q, long q_stride, int dim, int rot, int rot_dims, int neighbours, float magnitude,
+                                     const float* table, float* q_full, int rank, int heads, int n_tokens, void* stream) {
+  AXK_REQUIRE(q_stride >= (long)heads * (dim + rot), "latent_query_rope: rows %ld apart hold no %d heads of %d", q_stride, heads,
+              dim + rot);
   AXK_REQUIRE(n_tokens >= 0 && dim >= 0 && rot >= 0 && rank > 0 && heads > 0 && rot_dims % 2 == 0 && rot_dims <= rot,
               "latent_query_rope: bad sizes T=%d dim=%d rot=%d (%d rotated) rank=%d heads=%d", n_tokens, dim, rot, rot_dims,
               rank, heads);
   if (n_tokens == 0 || rot == 0) return 0;
-  latent_query_rope_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(q, dim, rot, rot_dims, table, q_full, rank, heads);
+  latent_query_rope_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(q, q_stride, dim, rot, rot_dims, neighbours, magnitude, table, q_full,
+                                                                      rank, heads);
   AXK_LAUNCH_CHECK("latent_query_rope");
   return 0;
 }
 
-// Few tokens (a decoding step) over a window: a wave per block of 64 positions, so that the blocks of a
-// token run side by side; the floats of the workspace this takes (0: the tokens' waves walk their
-// blocks themselves).  A window of w positions touches at most (w + 62) / 64 + 1 blocks.
-extern "C" long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window) {
-  if (!axk_latent_attention_uses_mfma(heads, rank, rot, page_size) || window <= 0) return 0;
-  const int blocks = (window + 62) / 64 + 1;
+// Few tokens (a decoding step): a wave per block of 64 positions, so that the blocks of a token run side
+// by side; the floats of the workspace this takes (0: the tokens' waves walk their blocks themselves).
+// A window of w positions touches at most (w + 62) / 64 + 1 blocks; without a window the caller says how
+// many positions the longest row of the step sees (`span`; 0: not known, no blocks side by side).
+static int latent_blocks_side_by_side(int window, int span) {
+  if (window > 0 && (span <= 0 || span > window)) return (window + 62) / 64 + 1;
+  return span > 0 ? (span + 63) / 64 : 0;
+}
+
+extern "C" long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window, int span) {
+  if (!axk_latent_attention_uses_mfma(heads, rank, rot, page_size)) return 0;
+  const int blocks = latent_blocks_side_by_side(window, span);
   if (blocks < 2 || (long)n_tokens * (heads / 16) >= 512) return 0;
   return (long)n_tokens * heads * blocks * (rank + 2);
 }
 
 extern "C" int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                                     const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads,
-                                    int rank, int rot, int page_size, int window, float scale, float* partial,
-                                    long partial_floats, void* stream) {
+                                    int rank, int rot, int page_size, int window, int span, float scale, const float* sink,
+                                    float* partial, long partial_floats, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && heads > 0 && rank > 0 && rot >= 0 && page_size > 0 && window >= 0,
               "latent_attention: bad sizes T=%d heads=%d rank=%d rot=%d page=%d window=%d", n_tokens, heads, rank, rot,
               page_size, window);
@@ -406,20 +432,20 @@ extern "C" int axk_latent_attention(const float* q_full, const void* cache, cons
   if (axk_latent_attention_uses_mfma(heads, rank, rot, page_size) && ((uintptr_t)q_full & 15) == 0 && ((uintptr_t)cache & 15) == 0 &&
       ((uintptr_t)o_lat & 15) == 0) {
     hipStream_t s = (hipStream_t)stream;
-    const long need = axk_latent_attention_workspace(n_tokens, heads, rank, rot, page_size, window);
+    const long need = axk_latent_attention_workspace(n_tokens, heads, rank, rot, page_size, window, span);
     AXK_REQUIRE(partial == nullptr || partial_floats >= need, "latent_attention: a workspace of %ld floats, %ld needed",
                 partial_floats, need);
     if (need == 0) partial = nullptr;
-    const int n_chunks = (window + 62) / 64 + 1;
+    const int n_chunks = latent_blocks_side_by_side(window, span);
     if (rank <= 64 && rank + rot <= 128)
       launch_latent_mfma<4, 4>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                               page_size, window, scale, partial, n_chunks, s);
+                               page_size, window, scale, sink, partial, n_chunks, s);
     else if (rank <= 128 && rank + rot <= 256)
       launch_latent_mfma<8, 8>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                               page_size, window, scale, partial, n_chunks, s);
+                               page_size, window, scale, sink, partial, n_chunks, s);
     else
       launch_latent_mfma<32, 20>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                                 page_size, window, scale, partial, n_chunks, s);
+                                 page_size, window, scale, sink, partial, n_chunks, s);
     AXK_LAUNCH_CHECK("latent_attention");
     return 0;
   }
@@ -428,7 +454,7 @@ extern "C" int axk_latent_attention(const float* q_full, const void* cache, cons
   const size_t lds = (size_t)(rank + rot) * LA_WAVES * sizeof(float);
   latent_attention_kernel<<<(unsigned)((items + LA_WAVES - 1) / LA_WAVES), LA_WAVES * 64, lds, (hipStream_t)stream>>>(
       q_full, (const elem_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-      page_size, window, scale);
+      page_size, window, scale, sink);
   AXK_LAUNCH_CHECK("latent_attention");
   return 0;
 }

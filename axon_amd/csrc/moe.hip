@@ -70,6 +70,68 @@ __global__ void route_topk_wave_kernel(const float* __restrict__ logits, int n_t
   if (lane < top) weights[(long)t * top + lane] = mine / sum;
 }
 
+// Scores that do not compete: s_e = sigmoid(z_e); the choice is made by s_e + correction_e (if given),
+// the weights come from s_e alone.  The experts form `groups` equal groups of neighbours; a group's
+// score is the sum of its two largest choice scores (of its one, if it has one expert), only experts
+// of the `keep` best groups can be chosen (of equal groups the lower), and among those the `top`
+// largest choice scores win (of equal ones the lower expert).  weights_k = s_k / (sum of the chosen s,
+// added in the order chosen, + 1e-20) * scale.  A wave per token: lane l holds experts l, l + 64, ...
+// (up to 1,024) and, for the groups' scores, walks group l (up to 64 groups).
+__global__ void route_scored_wave_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int n_tokens,
+                                         int n_experts, int top, int groups, int keep, float scale, int32_t* __restrict__ experts,
+                                         float* __restrict__ weights) {
+  const int t = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64, lane = threadIdx.x & 63;
+  if (t >= n_tokens) return;
+  const float* z = logits + (long)t * n_experts;
+  const int size = n_experts / groups;
+  unsigned long long kept = ~0ull;
+  if (groups > 1) {
+    float first = -INFINITY, second = -INFINITY;
+    if (lane < groups)
+      for (int e = lane * size; e < (lane + 1) * size; ++e) {
+        const float c = 1.0f / (1.0f + expf(-z[e])) + (correction ? correction[e] : 0.0f);
+        if (c > first) { second = first; first = c; }
+        else if (c > second) second = c;
+      }
+    const float mine = size > 1 ? first + second : first;
+    int ahead = 0;                                   // groups that rank before this lane's
+    for (int g = 0; g < groups; ++g) {
+      const float other = __shfl(mine, g, 64);
+      ahead += (other > mine || (other == mine && g < lane)) ? 1 : 0;
+    }
+    kept = __ballot(lane < groups && ahead < keep);
+  }
+  float choice[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int e = lane + 64 * i;
+    choice[i] = -INFINITY;
+    if (e < n_experts && (kept >> (e / size) & 1)) choice[i] = 1.0f / (1.0f + expf(-z[e])) + (correction ? correction[e] : 0.0f);
+  }
+  unsigned taken = 0;
+  float sum = 0.0f, mine = 0.0f;                     // lane k keeps the k-th score
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = lane + 64 * i;
+      if (e < n_experts && (kept >> (e / size) & 1) && !(taken >> i & 1) && (at == 0x7fffffff || choice[i] > best)) { best = choice[i]; at = e; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, 64);
+      const int other_at = __shfl_xor(at, off, 64);
+      if (other_at != 0x7fffffff && (at == 0x7fffffff || other > best || (other == best && other_at < at))) { best = other; at = other_at; }
+    }
+    if ((at & 63) == lane) taken |= 1u << (at >> 6);
+    const float s = 1.0f / (1.0f + expf(-z[at]));
+    sum += s;
+    if (lane == k % 64) { mine = s; experts[(long)t * top + k] = at; }
+  }
+  if (lane < top) weights[(long)t * top + lane] = (mine / (sum + 1e-20f)) * scale;
+}
+
 // One block.  pairs p = t top + k in expert order -> sorted [n_pairs], with the token of each
 // (sorted_tokens); tiles [.][3] = (expert, first place in sorted, count <= tile_rows), *n_tiles of them.
 // Which place a pair gets inside its expert's stretch is not fixed (atomic counters); no result
@@ -145,6 +207,20 @@ extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, 
   }
   route_topk_kernel<<<ceil_div(n_tokens, 64), 64, 0, (hipStream_t)stream>>>(logits, n_tokens, n_experts, top, experts, weights);
   AXK_LAUNCH_CHECK("route_topk");
+  return 0;
+}
+
+extern "C" int axk_route_scored(const float* logits, const float* correction, int n_tokens, int n_experts, int top, int groups,
+                                int keep, float scale, int32_t* experts, float* weights, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && n_experts > 0 && n_experts <= 1024 && top > 0 && top <= 64,
+              "route_scored: %d tokens, %d of %d experts (at most 64 of 1024)", n_tokens, top, n_experts);
+  AXK_REQUIRE(groups >= 1 && groups <= 64 && n_experts % groups == 0 && keep >= 1 && keep <= groups &&
+              (long)keep * (n_experts / groups) >= top,
+              "route_scored: %d of %d groups of %d experts for %d a token", keep, groups, n_experts / (groups > 0 ? groups : 1), top);
+  if (n_tokens == 0) return 0;
+  route_scored_wave_kernel<<<ceil_div(n_tokens, 4), 256, 0, (hipStream_t)stream>>>(logits, correction, n_tokens, n_experts, top, groups,
+                                                                                  keep, scale, experts, weights);
+  AXK_LAUNCH_CHECK("route_scored");
   return 0;
 }
 

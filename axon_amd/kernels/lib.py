@@ -80,9 +80,10 @@ _SIGNATURES = {
     "axk_clamped_glu": [c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_void_p],
     "axk_grouped_gemm_uses_mfma": [c_int, c_int, c_long, c_long],
     "axk_grouped_gemm": [c_void_p, c_int, c_long, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_long,
-                         c_void_p, c_void_p, c_long, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_void_p],
+                         c_void_p, c_void_p, c_long, c_int, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_void_p],
     "axk_route_topk": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "axk_route_scored": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p],
     "axk_route_max_tiles": [c_int, c_int, c_int],
     "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
@@ -91,11 +92,14 @@ _SIGNATURES = {
                         c_int, c_void_p],
     "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
                        c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
-    "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
-                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int,
+                           c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "axk_latent_query_rope": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                             c_int, c_int, c_float, c_void_p, c_long, c_void_p],
+                             c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
+    "axk_sum_norm": [c_void_p, c_float, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "axk_layernorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
+    "axk_softcap": [c_void_p, c_long, c_int, c_int, c_float, c_void_p],
     "axk_heads_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
                           c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                           c_int, c_void_p],
@@ -153,7 +157,7 @@ class Kernels:
             fn.restype = c_int
         self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
-        self.lib.axk_latent_attention_workspace.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
+        self.lib.axk_latent_attention_workspace.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_int]
         self.lib.axk_latent_attention_workspace.restype = ctypes.c_long
         self.lib.axk_masked_attention_workspace.argtypes = [c_int] * 9
         self.lib.axk_masked_attention_workspace.restype = ctypes.c_long
@@ -669,6 +673,44 @@ class Kernels:
                                           _ptr(x), _ptr(rounded), x.shape[0], x.shape[1], _stream()))
         return x
 
+    NORM_KINDS = {"rms": 0, "layer": 1}
+
+    def sum_norm(self, y: torch.Tensor, alpha: float, gain: torch.Tensor, eps: float, kind: str, x: torch.Tensor,
+                 rounded: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x = norm(alpha x + y) * gain, row by row (kind "rms" or "layer"); `rounded` also gets the new x in
+        the compute dtype."""
+        self._f32(y, "sum_norm y"); self._f32(x, "sum_norm x")
+        if y.shape != x.shape or y.dim() != 2 or gain.numel() != x.shape[1] or kind not in self.NORM_KINDS:
+            raise KernelError(f"sum_norm: y {tuple(y.shape)}, x {tuple(x.shape)}, a gain of {gain.numel()}, kind '{kind}'")
+        if rounded is not None:
+            self._elem(rounded, "sum_norm rounded")
+            if rounded.shape != x.shape or not rounded.is_contiguous():
+                raise KernelError(f"sum_norm: rounded {tuple(rounded.shape)} is not {tuple(x.shape)} contiguous")
+        self._check(self.lib.axk_sum_norm(_ptr(y), float(alpha), _ptr(gain), self._vec_flag(gain, "sum_norm gain"), float(eps),
+                                          self.NORM_KINDS[kind], _ptr(x), _ptr(rounded), x.shape[0], x.shape[1], _stream()))
+        return x
+
+    def layernorm(self, x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
+                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out = (x - mean) / sqrt(var + eps) * gain of float32 rows (`rows`: which of them)."""
+        self._f32(x, "layernorm x"); self._elem(out, "layernorm out")
+        n = x.shape[0]
+        if rows is not None:
+            self._i32(rows, "layernorm rows")
+            n = rows.numel()
+        if x.dim() != 2 or out.shape != (n, x.shape[1]) or not out.is_contiguous() or gain.numel() != x.shape[1]:
+            raise KernelError(f"layernorm: x {tuple(x.shape)}, out {tuple(out.shape)}, a gain of {gain.numel()}")
+        self._check(self.lib.axk_layernorm(_ptr(x), _ptr(rows), _ptr(gain), self._vec_flag(gain, "layernorm gain"), _ptr(out), n,
+                                           x.shape[1], float(eps), _stream()))
+        return out
+
+    def softcap(self, v: torch.Tensor, cap: float) -> torch.Tensor:
+        """v = cap tanh(v / cap) in place on float32 rows."""
+        if v.dtype != torch.float32 or not v.is_cuda or v.dim() != 2 or v.stride(1) != 1:
+            raise KernelError(f"softcap: {tuple(v.shape)} {v.dtype} with strides {v.stride()}")
+        self._check(self.lib.axk_softcap(_ptr(v), v.stride(0), v.shape[0], v.shape[1], float(cap), _stream()))
+        return v
+
     def round_rows(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         self._f32(x, "round_rows x"); self._elem(out, "round_rows out")
         if out.numel() != x.numel() or not out.is_contiguous():
@@ -705,16 +747,17 @@ class Kernels:
     # ------------------------------------------------------------------ grouped products
     def grouped_gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, x_group_stride: int, out_group_stride: int,
                      bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, glu=None, routed=None,
-                     rows: Optional[int] = None) -> torch.Tensor:
+                     rows: Optional[int] = None, gate_per_group: bool = False) -> torch.Tensor:
         """out[orow(r), g ogs + n] = epilogue(sum_k x[xrow(r), g xgs + k] w[g, n, k] + bias[g, n]).
 
         x [rows, >= g xgs + K] float32 or compute dtype, rows may be strided; w [G, N, K] (with `glu`
-        = (limit, alpha): [G, 2 N, K], gate rows then up rows) in the compute dtype; out float32 or
+        = (limit, alpha[, shift]): [G, 2 N, K], gate rows then up rows; out = g sigmoid(alpha g) (u + shift) with g
+        and u clamped by limit, shift 1 unless given; (inf, 1, 0) is silu(gate) up) in the compute dtype; out float32 or
         compute dtype.  Block-diagonal: every row meets every group.  `routed` = (tiles, n_tiles,
         max_tiles, x_rows, out_rows[, tile_rows]), int32 on the device: the listed rows (`rows` of them at
         most) meet the group their tile names; tile_rows (16, or 64: many rows a group) is what the list
         was made for.  `gate` (float32, out's shape): out is multiplied
-        by its sigmoid."""
+        by its sigmoid; with `gate_per_group` the gate holds one number a group, [rows, >= G]."""
         G, NW, K = w.shape
         N = NW // 2 if glu else NW
         self._elem(w, "grouped w")
@@ -731,8 +774,9 @@ class Kernels:
         if bias is not None and bias.numel() != G * NW:
             raise KernelError(f"grouped_gemm: a bias of {bias.numel()} for {G} x {NW}")
         if gate is not None:
-            if gate.dtype != torch.float32 or not gate.is_cuda or gate.dim() != 2 or gate.shape[0] != out.shape[0] or gate.stride(-1) != 1:
-                raise KernelError(f"grouped_gemm: gate {tuple(gate.shape)} for out {tuple(out.shape)}")
+            if gate.dtype != torch.float32 or not gate.is_cuda or gate.dim() != 2 or gate.shape[0] != out.shape[0] or gate.stride(-1) != 1 \
+                    or (gate_per_group and gate.shape[1] < G):
+                raise KernelError(f"grouped_gemm: gate {tuple(gate.shape)} for out {tuple(out.shape)} in {G} groups")
         tiles = n_tiles = x_rows = out_rows = None
         max_tiles, tile_rows = 0, 16
         if routed is not None:
@@ -743,12 +787,12 @@ class Kernels:
                     self._i32(t, "grouped_gemm routing")
             if x.shape[1] < K or out.shape[1] < N:
                 raise KernelError(f"grouped_gemm: x {tuple(x.shape)} / out {tuple(out.shape)} for {K} -> {N}")
-        limit, alpha = glu if glu else (0.0, 0.0)
+        limit, alpha, shift = (tuple(glu) + (1.0,))[:3] if glu else (0.0, 0.0, 0.0)
         self._check(self.lib.axk_grouped_gemm(
             _ptr(x), 1 if x.dtype == torch.float32 else 0, x.stride(0), x_group_stride, _ptr(x_rows), _ptr(w), _ptr(bias),
             self._vec_flag(bias, "grouped bias"), _ptr(out), 1 if out.dtype == torch.float32 else 0, out.stride(0),
-            out_group_stride, _ptr(out_rows), _ptr(gate), 0 if gate is None else gate.stride(0), 1 if glu else 0, float(limit),
-            float(alpha), _ptr(tiles), _ptr(n_tiles), int(max_tiles), int(tile_rows), M, N, K, G, _stream()))
+            out_group_stride, _ptr(out_rows), _ptr(gate), 0 if gate is None else gate.stride(0), 1 if gate_per_group else 0,
+            1 if glu else 0, float(limit), float(alpha), float(shift), _ptr(tiles), _ptr(n_tiles), int(max_tiles), int(tile_rows), M, N, K, G, _stream()))
         return out
 
     # ------------------------------------------------------------------ routing
@@ -758,6 +802,21 @@ class Kernels:
         if experts.shape != (T, top) or weights.shape != (T, top):
             raise KernelError(f"route_topk: {tuple(experts.shape)} / {tuple(weights.shape)} for {T} x {top}")
         self._check(self.lib.axk_route_topk(_ptr(logits), T, E, top, _ptr(experts), _ptr(weights), _stream()))
+
+    def route_scored(self, logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float,
+                     experts: torch.Tensor, weights: torch.Tensor) -> None:
+        """Sigmoid scores, the choice by score + correction among the `keep` best of `groups` groups of
+        neighbouring experts, weights the chosen scores over their sum, times scale (axk_route_scored)."""
+        self._f32(logits, "router logits"); self._i32(experts, "chosen experts"); self._f32(weights, "router weights")
+        T, E = logits.shape
+        if experts.shape != (T, top) or weights.shape != (T, top) or not logits.is_contiguous():
+            raise KernelError(f"route_scored: {tuple(experts.shape)} / {tuple(weights.shape)} for {T} x {top}")
+        if correction is not None:
+            self._f32(correction, "router correction")
+            if correction.numel() != E:
+                raise KernelError(f"route_scored: a correction of {correction.numel()} for {E} experts")
+        self._check(self.lib.axk_route_scored(_ptr(logits), _ptr(correction), T, E, top, int(groups), int(keep), float(scale),
+                                              _ptr(experts), _ptr(weights), _stream()))
 
     def route_max_tiles(self, n_pairs: int, n_experts: int, tile_rows: int = 16) -> int:
         return int(self.lib.axk_route_max_tiles(n_pairs, n_experts, tile_rows))
@@ -840,7 +899,7 @@ class Kernels:
 
     # ------------------------------------------------------------------ attention over a latent cache
     def latent_prepare(self, fused, q_at, q_rank, kv_at, rank, rot, rot_dims, q_gain, kv_gain, eps, table, positions, seq_rows,
-                       block_table, cache, page_size, cq, write_kv=True) -> None:
+                       block_table, cache, page_size, cq, write_kv=True, neighbours=False, magnitude=1.0) -> None:
         self._f32(fused, "latent fused"); self._f32(table, "rope table"); self._i32(positions, "positions")
         self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table"); self._elem(cache, "latent cache")
         T = positions.numel()
@@ -855,21 +914,27 @@ class Kernels:
         if kv_gain.numel() != rank:
             raise KernelError(f"latent_prepare: a gain of {kv_gain.numel()} for a latent of {rank}")
         self._check(self.lib.axk_latent_prepare(
-            _ptr(fused), fused.stride(0), q_at, q_rank, kv_at, rank, rot, rot_dims, _ptr(q_gain), self._vec_flag(q_gain, "q gain"),
+            _ptr(fused), fused.stride(0), q_at, q_rank, kv_at, rank, rot, rot_dims, 1 if neighbours else 0, float(magnitude),
+            _ptr(q_gain if q_rank else None), self._vec_flag(q_gain if q_rank else None, "q gain"),
             _ptr(kv_gain), self._vec_flag(kv_gain, "kv gain"), float(eps), _ptr(table), _ptr(positions), _ptr(seq_rows),
             _ptr(block_table), block_table.shape[-1], _ptr(cache), page_size, _ptr(cq if q_rank else None), T,
             1 if write_kv else 0, _stream()))
 
-    def latent_query_rope(self, q, dim, rot, rot_dims, table, q_full, rank, heads) -> None:
-        self._f32(q, "latent q"); self._f32(q_full, "latent q_full"); self._f32(table, "rope table")
+    def latent_query_rope(self, q, dim, rot, rot_dims, table, q_full, rank, heads, neighbours=False, magnitude=1.0) -> None:
+        """q: float32 [T, >= heads (dim + rot)], rows may be strided (a view into a wider product's rows)."""
+        self._f32(q_full, "latent q_full"); self._f32(table, "rope table")
         T = q.shape[0]
-        if q.shape != (T, heads * (dim + rot)) or q_full.shape != (T, heads * (rank + rot)):
+        if q.dtype != torch.float32 or not q.is_cuda or q.dim() != 2 or q.shape[1] < heads * (dim + rot) or q.stride(1) != 1 or q_full.shape != (T, heads * (rank + rot)) \
+                or not q_full.is_contiguous():
             raise KernelError(f"latent_query_rope: q {tuple(q.shape)}, q_full {tuple(q_full.shape)}")
-        self._check(self.lib.axk_latent_query_rope(_ptr(q), dim, rot, rot_dims, _ptr(table), _ptr(q_full), rank, heads, T,
-                                                   _stream()))
+        self._check(self.lib.axk_latent_query_rope(_ptr(q), q.stride(0), dim, rot, rot_dims, 1 if neighbours else 0, float(magnitude),
+                                                   _ptr(table), _ptr(q_full), rank, heads, T, _stream()))
 
     def latent_attention(self, q_full, cache, block_table, positions, seq_rows, o_lat, heads, rank, rot, page_size, window,
-                         scale) -> torch.Tensor:
+                         scale, sink=None, span: int = 0) -> torch.Tensor:
+        """`sink`: float32 [heads], a number a head whose exponential the softmax's denominator also holds;
+        `span`: the most positions a row of this step sees, where the caller knows it (attention without a
+        window then lets the blocks of a token's positions run side by side in steps of few tokens)."""
         self._f32(q_full, "latent q_full"); self._f32(o_lat, "latent o_lat"); self._elem(cache, "latent cache")
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
         T = positions.numel()
@@ -877,11 +942,15 @@ class Kernels:
             raise KernelError(f"latent_attention: q_full {tuple(q_full.shape)}, o_lat {tuple(o_lat.shape)} for {T} tokens")
         if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, 2 * rank + rot) or not cache.is_contiguous():
             raise KernelError(f"latent_attention: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {2 * rank + rot}]")
-        need = int(self.lib.axk_latent_attention_workspace(T, heads, rank, rot, page_size, int(window)))
+        if sink is not None:
+            self._f32(sink, "latent sink")
+            if sink.numel() != heads:
+                raise KernelError(f"latent_attention: {sink.numel()} sinks for {heads} heads")
+        need = int(self.lib.axk_latent_attention_workspace(T, heads, rank, rot, page_size, int(window), int(span)))
         partial = torch.empty(need, dtype=torch.float32, device=o_lat.device) if need else None
         self._check(self.lib.axk_latent_attention(_ptr(q_full), _ptr(cache), _ptr(block_table), block_table.shape[-1],
                                                   _ptr(positions), _ptr(seq_rows), _ptr(o_lat), T, heads, rank, rot, page_size,
-                                                  int(window), float(scale), _ptr(partial), need, _stream()))
+                                                  int(window), int(span), float(scale), _ptr(sink), _ptr(partial), need, _stream()))
         return o_lat
 
     # ------------------------------------------------------------------ attention with maps, masks and bent scores

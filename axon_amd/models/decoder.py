@@ -10,7 +10,7 @@ import torch
 
 from ..cache.manager import GroupPlan
 from ..config.base import ConfigError, ModelConfig
-from ..parts.base import CacheBinding, TensorDecl, build_block, build_part
+from ..parts.base import ROUNDED_STREAM, CacheBinding, TensorDecl, build_block, build_part
 
 
 @dataclass
@@ -138,6 +138,7 @@ class DecoderModel:
             block = self.blocks[run.layer]
             if run.enter is not None:
                 self.entries[run.enter].forward(ctx, x, ctx.shared["embedding_output"])
+                ctx.shared[ROUNDED_STREAM] = None        # what a block left of the stream it wrote is no longer the stream
             following = None
             if i + 1 < end and self.order[i + 1].enter is None:     # a rewritten stream is normed by its own pass
                 after = self.blocks[self.order[i + 1].layer]

@@ -221,6 +221,11 @@ class StreamEntry(Part):
         raise NotImplementedError
 
 
+# A block may leave in ctx.shared, under this key, (the stream, its rows in the compute dtype) for the
+# block after it; whatever rewrites the stream between two blocks sets the value to None.
+ROUNDED_STREAM = "rounded rows of the stream"
+
+
 class Block(Part):
     """An arrangement: built from the layer's parts, not from a spec of its own.
 

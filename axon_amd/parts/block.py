@@ -11,7 +11,7 @@ from typing import List
 import torch
 
 from ..config.base import ConfigError
-from .base import Block, CacheBinding, TensorDecl, register_block
+from .base import ROUNDED_STREAM, Block, CacheBinding, TensorDecl, register_block
 
 # A norm behind a product whose kernel holds the finished rows anyway can be written by that
 # kernel, and a norm before a product of few rows can be worked out inside that product (the same
@@ -154,6 +154,56 @@ class SublayerNormBlock(Block):
         k.norm_add(y, self.norm2.gain, self.norm2.eps, self.mult, x)
 
 
+class PostNormBlock(Block):
+    """x <- norm1(alpha x + mixer(x)); x <- norm2(alpha x + feed_forward(x)): the norms sit behind the
+    sums, the sublayers read the stream itself (rounded to the compute dtype for their products), and
+    a layer may have no feed-forward (it then has no second norm).  The scaling, the sum and the norm
+    are one 32-bit pass over the sublayer's 32-bit output, which also leaves the new rows rounded for
+    the next sublayer, the next block's too.  The norms are RMS or layer norms (a gain, an eps and a
+    `kind`); `stream_alpha` comes with the norm's parameters."""
+    graph_safe = True
+    norm1_name = "norm1"
+    norm2_name = "norm2"
+
+    def __init__(self, norm_factory, mixer, feed_forward, prefix):
+        super().__init__(norm_factory, mixer, feed_forward, prefix)
+        self.norm1 = norm_factory(self.norm1_name)
+        self.norm2 = norm_factory(self.norm2_name) if feed_forward is not None else None
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not all(hasattr(norm, a) for a in ("gain", "eps", "kind")):
+                raise ConfigError("a norm behind a sum is an RMS norm or a layer norm (a gain, an eps and a kind)")
+        self.alpha = float(self.norm1.params.get("stream_alpha", 1.0))
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    def tensors(self) -> List[TensorDecl]:
+        return [d for p in self.parts() for d in p.tensors()]
+
+    def load(self, store, rt) -> None:
+        for part in self.parts():
+            part.load(store, rt)
+
+    _run = staticmethod(SublayerNormBlock._run)
+
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
+        k, rt = ctx.rt.k, ctx.rt
+        exact = rt.dtype == torch.float32            # the 32-bit path: the sublayers read x as it is
+        h = x
+        if not exact:
+            left = ctx.shared.get(ROUNDED_STREAM)    # the block before left the rows it wrote, rounded
+            h = left[1] if left is not None and left[0] is x else k.round_rows(x, ctx.ws.take(tuple(x.shape), rt.dtype))
+        y = ctx.ws.take(tuple(x.shape), torch.float32)
+        self._run(self.mixer, ctx, y, binding, h)
+        h = None if exact else ctx.ws.take(tuple(x.shape), rt.dtype)
+        k.sum_norm(y, self.alpha, self.norm1.gain, self.norm1.eps, self.norm1.kind, x, h)
+        if self.feed_forward is not None:
+            self._run(self.feed_forward, ctx, y, x if exact else h)
+            k.sum_norm(y, self.alpha, self.norm2.gain, self.norm2.eps, self.norm2.kind, x, h)
+        ctx.shared[ROUNDED_STREAM] = None if exact else (x, h)
+
+
 register_block("prenorm", PreNormBlock)
 register_block("prenorm_short_names", ShortNamedPreNormBlock)
 register_block("sublayer_norm", SublayerNormBlock)
+register_block("postnorm", PostNormBlock)

@@ -52,6 +52,7 @@ class LMHead(Part):
         self.name = prefix + params["tensor"]
         self.tied_to = params.get("tied_to")
         self.tied = bool(params.get("tied", False))
+        self.softcap = float(params.get("softcap", 0.0))      # > 0: logits = cap tanh(logits / cap)
         self.weight = None
         self.source_name = None      # the tensor the head was loaded from
 
@@ -79,7 +80,10 @@ class LMHead(Part):
         """h: [rows, hidden] in the compute dtype -> float32 logits [rows, vocab]."""
         if out is None:
             out = torch.empty((h.shape[0], self.vocab), dtype=torch.float32, device=h.device)
-        return ctx.rt.k.gemm(h, self.weight, out, None, MODE_STORE_F32)
+        ctx.rt.k.gemm(h, self.weight, out, None, MODE_STORE_F32)
+        if self.softcap > 0.0:
+            ctx.rt.k.softcap(out, self.softcap)
+        return out
 
 
 register_embedding("token_embedding", TokenEmbedding)

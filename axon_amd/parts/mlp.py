@@ -3,7 +3,7 @@
 act = (g / (1 + exp(-g))) * u (src/vmath.rs:128-132), no biases (src/model.rs:3043-3055).
 gate and up run as one product over a fused [2 ffn, hidden] matrix whose epilogue applies the
 activation, so the two halves never travel through memory.  Parameters:
-`hidden_size`, `intermediate_size`.
+`hidden_size`, `intermediate_size`, `names` (scope "mlp.", gate, up, down, suffix ".weight").
 """
 from __future__ import annotations
 
@@ -16,13 +16,15 @@ from .base import FeedForward, PrecedingNorm, TensorDecl, register_feed_forward
 
 class SwiGLUMLP(FeedForward):
     graph_safe = True
+    stores_output = True
+
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.hidden = int(params["hidden_size"])
         self.ffn = int(params["intermediate_size"])
         names = params.get("names", {})
         base = prefix + names.get("scope", "mlp.")
-        self.n = {k: base + names.get(k, k + "_proj") + ".weight" for k in ("gate", "up", "down")}
+        self.n = {k: base + names.get(k, k + "_proj") + names.get("suffix", ".weight") for k in ("gate", "up", "down")}
         self.w_gate_up = self.w_down = None
 
     def tensors(self) -> List[TensorDecl]:
@@ -41,7 +43,7 @@ class SwiGLUMLP(FeedForward):
         return (isinstance(self.w_gate_up, PackedMatrix)
                 and ctx.rt.k.gemm_normed_ok(ctx.n_tokens, self.ffn, self.hidden, gated=True))
 
-    def forward(self, ctx, h, residual, following=None) -> None:
+    def forward(self, ctx, h, residual, following=None, accumulate: bool = True) -> None:
         k = ctx.rt.k
         act = ctx.ws.take((h.shape[0], self.ffn), ctx.rt.dtype)
         if isinstance(h, PrecedingNorm) and not k.gemm_normed_ok(h.shape[0], self.ffn, self.hidden, gated=True, gain=h.gain):
@@ -50,6 +52,9 @@ class SwiGLUMLP(FeedForward):
             k.gemm_normed_glu(h.rows, h.gain, h.eps, self.w_gate_up, act)
         else:
             k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)   # silu(gate h) * up h, in the product's epilogue
+        if not accumulate:          # the output itself, for a block that sums and norms on its own
+            k.gemm(act, self.w_down, residual, None, MODE_STORE_F32)
+            return
         k.gemm(act, self.w_down, residual, None, MODE_ADD_F32,
                following_norm=None if following is None else following.as_argument())
 

@@ -1,5 +1,9 @@
-"""A mixture of experts: each token goes through the `top` experts its router logits rank first,
-weighted by the softmax over those logits alone; a shared expert, if any, sees every token.
+"""A mixture of experts: each token goes through the `top` experts its router ranks first; a shared
+expert, if any, sees every token.  Two routers: "softmax" (the default): the largest logits, weighted by
+the softmax over those logits alone; "sigmoid": scores s = sigmoid(logits) that do not compete, the
+choice made by s + a stored correction among the experts of the `keep` best of `groups` equal groups of
+neighbours (a group's score: the sum of its two largest choice scores), weighted by s over the sum of
+the chosen s, times `scale`.
 
 Router logits are 32-bit (Wr h with h in the compute dtype).  An expert is a gated unit with
 clamps: g = min(Wgate h, limit), u = clamp(Wup h, -limit, limit), out = Wdown (g sigmoid(alpha g)
@@ -9,11 +13,15 @@ over the list; a token's rows are then added in the order of its router's rankin
 an expert (a long prompt) the list is made in tiles of 64 rows, which the grouped product takes
 through LDS: the same chains and bits as the tiles of 16 of a short step.
 
-Parameters: `hidden_size`, `experts`, `top`, `ff`, `limit`, `alpha` (default 1.702), `shared`
-(None, or {"ff", "limit"}), `names` (scope "mlp.", router, expert "e{}.", shared "shared.").
+Parameters: `hidden_size`, `experts`, `top`, `ff`, `limit` (None: no clamps), `alpha` (default 1.702),
+`shift` (default 1: the unit is g sigmoid(alpha g) (u + shift); no clamps, alpha 1 and shift 0 make it
+silu(gate) up), `router` (None, or {"scores": "sigmoid", "correction": bool, "groups", "keep", "scale"}),
+`shared` (None, or {"ff", "limit"}), `names` (scope "mlp.", router, correction, expert "e{}.", shared
+"shared.").
 """
 from __future__ import annotations
 
+import math
 from typing import List
 
 import torch
@@ -31,12 +39,30 @@ class RoutedExperts(FeedForward):
         super().__init__(params, prefix)
         p = params
         self.hidden, self.n_experts, self.top = int(p["hidden_size"]), int(p["experts"]), int(p["top"])
-        self.ff, self.limit, self.alpha = int(p["ff"]), float(p["limit"]), float(p.get("alpha", 1.702))
+        self.ff, self.alpha, self.shift = int(p["ff"]), float(p.get("alpha", 1.702)), float(p.get("shift", 1.0))
+        self.limit = math.inf if p.get("limit") is None else float(p["limit"])
         if not 1 <= self.top <= self.n_experts:
             raise ConfigError(f"{self.top} of {self.n_experts} experts a token")
         names = p.get("names", {})
         self.base = prefix + names.get("scope", "mlp.")
         self.router_name = self.base + names.get("router", "router")
+        router = dict(p.get("router") or {})
+        self.scores = router.get("scores", "softmax")
+        if self.scores not in ("softmax", "sigmoid"):
+            raise ConfigError(f"a router with '{self.scores}' scores is not known (softmax, sigmoid)")
+        self.groups, self.keep = int(router.get("groups", 1)), int(router.get("keep", 1))
+        self.route_scale = float(router.get("scale", 1.0))
+        self.correction_name = self.base + names.get("correction", "correction") if router.get("correction") else None
+        self.correction = None
+        if self.scores == "sigmoid":
+            if self.n_experts > 1024 or self.top > 64 or self.groups > 64:
+                raise ConfigError(f"the sigmoid router takes up to 1024 experts in up to 64 groups and up to 64 a token, "
+                                  f"not {self.top} of {self.n_experts} in {self.groups}")
+            if self.groups < 1 or self.n_experts % self.groups or not 1 <= self.keep <= self.groups \
+                    or self.keep * (self.n_experts // self.groups) < self.top:
+                raise ConfigError(f"{self.keep} of {self.groups} groups of {self.n_experts} experts cannot give {self.top} a token")
+        elif router:
+            raise ConfigError("groups, a correction and a scale belong to the router with sigmoid scores")
         self.expert_scope = names.get("expert", "e{}.")
         self.shared = None
         if p.get("shared"):
@@ -51,6 +77,8 @@ class RoutedExperts(FeedForward):
 
     def tensors(self) -> List[TensorDecl]:
         t = [TensorDecl(self.router_name, (self.n_experts, self.hidden))]
+        if self.correction_name is not None:
+            t.append(TensorDecl(self.correction_name, (self.n_experts,), "bias"))
         for e in range(self.n_experts):
             t += [TensorDecl(self._expert(e, "gate"), (self.ff, self.hidden)), TensorDecl(self._expert(e, "up"), (self.ff, self.hidden)),
                   TensorDecl(self._expert(e, "down"), (self.hidden, self.ff))]
@@ -58,6 +86,8 @@ class RoutedExperts(FeedForward):
 
     def load(self, store, rt) -> None:
         self.w_router = rt.k.prepare_weight(store.matrix(self.router_name))
+        if self.correction_name is not None:
+            self.correction = store.vector(self.correction_name).float().contiguous()
         E = self.n_experts
         # every expert's gate rows, then its up rows: [experts, 2 ff, hidden]; and [experts, hidden, ff]
         self.w_gate_up = torch.empty((E, 2 * self.ff, self.hidden), dtype=rt.dtype, device=rt.device)
@@ -77,7 +107,10 @@ class RoutedExperts(FeedForward):
         logits = ctx.ws.take((T, E), torch.float32)
         k.gemm(h, self.w_router, logits, None, MODE_STORE_F32)
         chosen, weights = ctx.ws.take((T, top), i32), ctx.ws.take((T, top), torch.float32)
-        k.route_topk(logits, top, chosen, weights)
+        if self.scores == "sigmoid":
+            k.route_scored(logits, self.correction, top, self.groups, self.keep, self.route_scale, chosen, weights)
+        else:
+            k.route_topk(logits, top, chosen, weights)
         P = T * top
         tile_rows = 64 if P >= 32 * E else 16          # many rows an expert: tiles of 64 rows through LDS (the same bits)
         max_tiles = k.route_max_tiles(P, E, tile_rows)
@@ -85,7 +118,7 @@ class RoutedExperts(FeedForward):
         tiles, n_tiles = ctx.ws.take((3 * max_tiles,), i32), ctx.ws.take((1,), i32)
         k.route_sort(chosen, E, pairs, tokens, tiles, n_tiles, tile_rows=tile_rows)
         act = ctx.ws.take((P, self.ff), ctx.rt.dtype)
-        k.grouped_gemm(h, self.w_gate_up, act, x_group_stride=0, out_group_stride=0, glu=(self.limit, self.alpha),
+        k.grouped_gemm(h, self.w_gate_up, act, x_group_stride=0, out_group_stride=0, glu=(self.limit, self.alpha, self.shift),
                        routed=(tiles, n_tiles, max_tiles, tokens, pairs, tile_rows), rows=P)
         rows = ctx.ws.take((P, self.hidden), torch.float32)
         k.grouped_gemm(act, self.w_down, rows, x_group_stride=0, out_group_stride=0,

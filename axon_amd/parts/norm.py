@@ -1,4 +1,4 @@
-"""RMSNorm: rows of the 32-bit residual stream, normalised into the compute dtype.
+"""Norms: rows of the 32-bit residual stream, normalised into the compute dtype (RMSNorm, LayerNorm).
 
 out = (x * 1/sqrt(mean(x^2) + eps)) * gain (src/model.rs:3888-3898).  Parameters: `size`,
 `eps`, `tensor` (the gain's name under the part's prefix), `offset` (default 0: the gain is
@@ -16,6 +16,7 @@ from .base import FollowingNorm, Norm, PrecedingNorm, TensorDecl, register_norm
 
 class RMSNorm(Norm):
     graph_safe = True
+    kind = "rms"         # what a kernel that norms on the way (the sum before a norm, say) is told
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.size = int(params["size"])
@@ -49,4 +50,33 @@ class RMSNorm(Norm):
         return PrecedingNorm(self, x)
 
 
+class LayerNorm(Norm):
+    """out = (x - mean x) / sqrt(var x + eps) * gain, the variance the mean of the squared deviations;
+    a gain and no bias.  Parameters: `size`, `eps`, `tensor`.  It offers itself to no product (the
+    products' norms are RMS norms): it runs as a pass of its own, or inside the pass of a block that
+    norms behind its sums."""
+    graph_safe = True
+    kind = "layer"
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.name = prefix + params.get("tensor", "weight")
+        self.gain = None
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.name, (self.size,), "gain")]
+
+    def load(self, store, rt) -> None:
+        self.gain = store.vector(self.name)
+
+    def forward(self, ctx, x, out=None, rows: Optional["torch.Tensor"] = None):
+        n = x.shape[0] if rows is None else rows.numel()
+        if out is None:
+            out = ctx.ws.take((n, self.size), ctx.rt.dtype)
+        return ctx.rt.k.layernorm(x, self.gain, self.eps, out, rows)
+
+
 register_norm("rmsnorm", RMSNorm)
+register_norm("layernorm", LayerNorm)
