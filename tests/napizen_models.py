@@ -3,7 +3,9 @@ between the layers of a model (query/key size against value size, latent against
 (one head, one expert a token, groups of one expert, no stretch of the stream, no scale), widths that
 no matrix-core product takes and heads in sixteens that the matrix-core attention takes, fewer rotated
 dims than the rotated part holds, frequencies ramped and not, and weights drawn so that the mechanisms
-matter: sinks of the size of the scores, corrections large enough to turn a choice score negative."""
+matter: sinks of the size of the scores, corrections large enough to turn a choice score negative.  The
+attention's `scale` keeps a score's spread near 3 under these weights: 16 bits of cache cannot carry
+weights much sharper."""
 import json
 import os
 
@@ -63,9 +65,9 @@ MODELS = {
         eps=1e-4, alpha=2.5, scale=9.0, softcap=50.0), page=64, seed=5),
     # one head, a rotated part of two dims, pages of 16, two groups of which one stays, three of its four experts
     "D": dict(cfg=config(80, 140, [
-        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.7), moe(8, 3, 24, (2, 1), 1.5)),
-        layer(att(heads=5, dim=8, rot_dim=8, vdim=16, kv_rank=12, base=10000.0, scaling=(16.0, 8, 2.0, 1.0), scale=0.8), dense(96)),
-        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.7), moe(8, 3, 24, (2, 1), 1.5))],
+        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.5)),
+        layer(att(heads=5, dim=8, rot_dim=8, vdim=16, kv_rank=12, base=10000.0, scaling=(16.0, 8, 2.0, 1.0), scale=0.35), dense(96)),
+        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.5))],
         eps=1e-6, alpha=0.8, scale=2.0, softcap=15.0), page=16, seed=12),
 }
 

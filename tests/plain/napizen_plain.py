@@ -137,39 +137,49 @@ def choose_experts(scores, correction, top, groups, keep):
     return sorted(allowed, key=lambda e: (-choice[e], e))[:top]
 
 
-def routed_ff(W, p, c, h):
+def routed_ff(W, p, c, h, forced=None, slack=0.0):
+    """forced: for every token the experts another implementation chose.  They are taken instead of this
+    one's own choice, after a check that they are a choice one may arrive at: the one made when each
+    of them scores `slack` higher (a close call that rounding decides the other way)."""
     r = c["router"]
     s = sigma(h @ W[p + "router"].T)
     groups = r.get("groups") or {"count": 1, "keep": 1}
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         chosen = choose_experts(s[t], W[p + "correction"], r["top"], groups["count"], groups["keep"])
+        if forced is not None and sorted(forced[t]) != sorted(chosen):
+            lifted = s[t].clone()
+            lifted[list(forced[t])] += slack
+            close = choose_experts(lifted, W[p + "correction"], r["top"], groups["count"], groups["keep"])
+            assert sorted(close) == sorted(forced[t]), f"{p} token {t}: {forced[t]} is no close call of {chosen}"
+            chosen = list(forced[t])
         total = sum(s[t, e] for e in chosen) + 1e-20
         for e in chosen:
             out[t] += s[t, e] / total * r["scale"] * gated_unit(W, f"{p}e{e}.", h[t:t + 1])[0]
     return out
 
 
-def feed_forward(W, p, c, h):
-    return gated_unit(W, p, h) if c["kind"] == "dense" else routed_ff(W, p, c, h)
+def feed_forward(W, p, c, h, forced=None, slack=0.0):
+    return gated_unit(W, p, h) if c["kind"] == "dense" else routed_ff(W, p, c, h, forced, slack)
 
 
 # --------------------------------------------------------------------------- the model
-def residual_stream(cfg, W, tokens, after_every_layer=None):
+def residual_stream(cfg, W, tokens, after_every_layer=None, forced=None, slack=0.0):
+    """forced: {layer: the experts chosen for every token} for layers with experts (see routed_ff)."""
     eps, alpha = cfg["norm"]["eps"], cfg.get("postln_alpha", 1.0)
     x = W["embed"][torch.as_tensor(tokens)] * cfg.get("embedding", {}).get("scale", 1.0)
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
         x = layer_norm(alpha * x + latent_attention(W, p + "mix.", layer["mixer"], x, eps), W[p + "norm1"], eps)
         if layer.get("mlp") is not None:
-            x = layer_norm(alpha * x + feed_forward(W, p + "mlp.", layer["mlp"], x), W[p + "norm2"], eps)
+            x = layer_norm(alpha * x + feed_forward(W, p + "mlp.", layer["mlp"], x, (forced or {}).get(i), slack), W[p + "norm2"], eps)
         if after_every_layer is not None:
             after_every_layer.append(x.clone())
     return x
 
 
-def forward_logits(cfg, W, tokens):
-    x = residual_stream(cfg, W, tokens)
+def forward_logits(cfg, W, tokens, forced=None, slack=0.0):
+    x = residual_stream(cfg, W, tokens, None, forced, slack)
     z = layer_norm(x, W["final.norm"], cfg["norm"]["eps"]) @ W["head"].T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(z / cap) if cap else z
