@@ -126,13 +126,44 @@ def _figalorn_sizes(width, heads, kv_heads, ff, window, chunk):
             "loop": {"start": 0, "stop": 1, "times": 2}, "norm": {"eps": 1e-6}, "vocab": 32000, "width": width}
 
 
+# --design napizen: four layers of latent attention without a window (a sink in the softmax, a gate a head, queries from
+# one matrix), the first with a gated feed-forward, the others with experts chosen by sigmoid scores in groups; layer
+# norms behind the sums.  Beside it the closest design the engine has at the same sizes, Pikesun's latent attention
+# (no window either) with as many experts of the same width (its two-matrix feed-forward 1.5 times as wide: the same
+# weights), and the dense decoder of equal width.
+def _napizen_sizes(width, heads, experts, top, expert_ff, dense_ff, groups, keep):
+    att = {"type": "latent_attention", "mixer": {
+        "heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+        "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": groups, "keep": keep}},
+           "expert": {"ff": expert_ff}}
+    layers = [dict(att, mlp={"kind": "dense", "ff": dense_ff})] + [dict(att, mlp=moe)] * 3
+    return {"architecture": "Napizen", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-6},
+            "postln_alpha": 1.0, "logit_softcap": 30.0, "vocab": 32000, "width": width}
+
+
+def _pikesun_attention_sizes(width, heads, q_rank, experts, top, expert_ff, dense_ff):
+    att = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+                                                 "q_rank": q_rank, "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff, "limit": 7.0}}
+    layers = [dict(att, mlp={"kind": "dense", "ff": dense_ff * 3 // 2})] + [dict(att, mlp=moe)] * 3
+    return {"architecture": "Pikesun", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-6},
+            "residual_mult": 1.0, "vocab": 32000, "width": width}
+
+
+# design -> size -> the models measured side by side, the design's own first
 DESIGN_SIZES = {
     "pikesun": {
-        "2048": (_pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024), _qwen_sizes(2048, 16, 2, 5632)),
-        "4096": (_pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048), _qwen_sizes(4096, 32, 8, 11008))},
+        "2048": [("pikesun", _pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024)), ("qwen2", _qwen_sizes(2048, 16, 2, 5632))],
+        "4096": [("pikesun", _pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048)), ("qwen2", _qwen_sizes(4096, 32, 8, 11008))]},
     "figalorn": {
-        "2048": (_figalorn_sizes(2048, 16, 2, 5632, 1024, 1536), _qwen_sizes(2048, 16, 2, 5632)),
-        "4096": (_figalorn_sizes(4096, 32, 8, 11008, 2048, 8192), _qwen_sizes(4096, 32, 8, 11008))},
+        "2048": [("figalorn", _figalorn_sizes(2048, 16, 2, 5632, 1024, 1536)), ("qwen2", _qwen_sizes(2048, 16, 2, 5632))],
+        "4096": [("figalorn", _figalorn_sizes(4096, 32, 8, 11008, 2048, 8192)), ("qwen2", _qwen_sizes(4096, 32, 8, 11008))]},
+    "napizen": {
+        "2048": [("napizen", _napizen_sizes(2048, 16, 32, 4, 704, 5632, 4, 2)),
+                 ("pikesun", _pikesun_attention_sizes(2048, 16, 768, 32, 4, 704, 5632)), ("qwen2", _qwen_sizes(2048, 16, 2, 5632))],
+        "4096": [("napizen", _napizen_sizes(4096, 32, 64, 6, 1408, 11008, 8, 4)),
+                 ("pikesun", _pikesun_attention_sizes(4096, 32, 1536, 64, 6, 1408, 11008)), ("qwen2", _qwen_sizes(4096, 32, 8, 11008))]},
 }
 
 
@@ -146,11 +177,11 @@ def design(args, torch) -> int:
     out = {"design": args.design, "dtype": args.dtype, "prompt_tokens": T, "batch": batch, "data": "synthetic (random weights)",
            "sizes": {}}
     gen = torch.Generator().manual_seed(0)
-    for size, pair in DESIGN_SIZES[args.design].items():
+    for size, models in DESIGN_SIZES[args.design].items():
         if args.design_size and size != args.design_size:
             continue
         row = out["sizes"][size] = {}
-        for label, cfg in zip((args.design, "qwen2"), pair):
+        for label, cfg in models:
             llm = axon_amd.load(cfg, dtype=args.dtype, random_seed=0, init_std=0.02, page_size=64,
                                 num_pages=(batch + 1) * (-(-(T + steps + args.warmup + 80) // 64)) + 8, max_seqs=batch + 1,
                                 max_batch_tokens=T, max_seq_len=T + steps + args.warmup + 80)
@@ -197,7 +228,7 @@ def design(args, torch) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default="", choices=["", "pikesun", "figalorn"], help="instead of the headline benchmark: prefill and "
+    ap.add_argument("--design", default="", choices=["", "pikesun", "figalorn", "napizen"], help="instead of the headline benchmark: prefill and "
                     "decoding of this design at sizes that resemble real models' layers, beside the dense decoder of equal size")
     ap.add_argument("--design-size", default="", help="with --design: only this size (2048 or 4096)")
     ap.add_argument("--gpus", type=int, default=1)

@@ -93,8 +93,10 @@ class RouterLog:
 
 def run_schedule(eng, name, seqs, schedule):
     """schedule: steps of [(request, tokens)]; every position's logits are asked for.  A request
-    ends with its last token.  Returns ({request: [len, vocab]}, {request: {layer: chosen experts by position}})."""
-    routed = [i for i, L in enumerate(MODELS[name]["cfg"]["layers"]) if L.get("mlp") and L["mlp"]["kind"] == "moe"]
+    ends with its last token.  `name`: one of MODELS, or a configuration.  Returns ({request: [len, vocab]},
+    {request: {layer: chosen experts by position}})."""
+    cfg = MODELS[name]["cfg"] if isinstance(name, str) else name
+    routed = [i for i, L in enumerate(cfg["layers"]) if L.get("mlp") and L["mlp"]["kind"] == "moe"]
     at = {r: 0 for r in seqs}
     got = {r: [] for r in seqs}
     chose = {r: {i: [] for i in routed} for r in seqs}
