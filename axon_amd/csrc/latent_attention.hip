@@ -320,24 +320,33 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
 
 // o_lat[row, :] = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) l_c over a row's blocks in ascending order
 // (M the largest m_c; a block that saw nothing has l = 0 and weighs nothing).  One block per (token,
-// head): the blocks' weights once into LDS, then a thread a dim.  With a sink, M is at least the head's
-// sink and the sum of the weights holds exp(sink - M) as well.
-__global__ void __launch_bounds__(128)
+// head): the blocks' (m, l) once into LDS, all loads in flight together, their weights from there, then
+// a thread a dim whose chain over the blocks has eight loads in flight.  With a sink, M is at least the
+// head's sink and the sum of the weights holds exp(sink - M) as well.
+__global__ void __launch_bounds__(512)
 latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks,
                              const float* __restrict__ sink, int heads) {
-  extern __shared__ float weight[];
+  extern __shared__ float fold_lds[];
+  float* weight = fold_lds;
+  float* ms = fold_lds + n_chunks;
+  float* ls = ms + n_chunks;
   const float* src = partial + (long)blockIdx.x * n_chunks * (rank + 2);
+  for (int c = threadIdx.x; c < n_chunks; c += blockDim.x) {
+    ms[c] = src[(long)c * (rank + 2) + rank];
+    ls[c] = src[(long)c * (rank + 2) + rank + 1];
+  }
+  __syncthreads();
   float M = sink ? sink[blockIdx.x % heads] : -INFINITY;
   for (int c = 0; c < n_chunks; ++c)
-    if (src[(long)c * (rank + 2) + rank + 1] > 0.0f) M = fmaxf(M, src[(long)c * (rank + 2) + rank]);
-  for (int c = threadIdx.x; c < n_chunks; c += blockDim.x)
-    weight[c] = src[(long)c * (rank + 2) + rank + 1] > 0.0f ? expf(src[(long)c * (rank + 2) + rank] - M) : 0.0f;
+    if (ls[c] > 0.0f) M = fmaxf(M, ms[c]);
+  for (int c = threadIdx.x; c < n_chunks; c += blockDim.x) weight[c] = ls[c] > 0.0f ? expf(ms[c] - M) : 0.0f;
   __syncthreads();
   float L = sink ? expf(sink[blockIdx.x % heads] - M) : 0.0f;
-  for (int c = 0; c < n_chunks; ++c) L = fmaf(weight[c], src[(long)c * (rank + 2) + rank + 1], L);
+  for (int c = 0; c < n_chunks; ++c) L = fmaf(weight[c], ls[c], L);
   const float inv = 1.0f / L;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float o = 0.0f;
+#pragma unroll 8
     for (int c = 0; c < n_chunks; ++c) o = fmaf(weight[c], src[(long)c * (rank + 2) + d], o);
     o_lat[(long)blockIdx.x * rank + d] = o * inv;
   }
@@ -354,7 +363,8 @@ static void launch_latent_mfma(const float* q_full, const void* cache, const int
       q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
       window, scale, sink, partial, n_chunks);
   if (partial)
-    latent_attention_fold_kernel<<<n_tokens * heads, 128, n_chunks * sizeof(float), stream>>>(partial, o_lat, rank, n_chunks, sink, heads);
+    latent_attention_fold_kernel<<<n_tokens * heads, min(512, (rank + 63) / 64 * 64), 3 * n_chunks * sizeof(float), stream>>>(
+        partial, o_lat, rank, n_chunks, sink, heads);
 }
 #endif
 

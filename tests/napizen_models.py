@@ -62,13 +62,13 @@ MODELS = {
     "C": dict(cfg=config(64, 257, [
         layer(att(heads=32, dim=8, rot_dim=32, vdim=8, kv_rank=32, dims=16, base=500.0, scale=0.4), moe(8, 2, 32, (8, 3), 1.0)),
         layer(att(heads=16, dim=16, rot_dim=64, vdim=24, kv_rank=192, base=10000.0, scaling=(2.0, 32, 4.0, 0.5), scale=0.25), moe(5, 1, 16, (1, 1), 0.5))],
-        eps=1e-4, alpha=2.5, scale=9.0, softcap=50.0), page=64, seed=5),
+        eps=1e-4, alpha=2.2, scale=9.0, softcap=50.0), page=64, seed=5),
     # one head, a rotated part of two dims, pages of 16, two groups of which one stays, three of its four experts
     "D": dict(cfg=config(80, 140, [
-        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.5)),
+        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.25)),
         layer(att(heads=5, dim=8, rot_dim=8, vdim=16, kv_rank=12, base=10000.0, scaling=(16.0, 8, 2.0, 1.0), scale=0.35), dense(96)),
-        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.5))],
-        eps=1e-6, alpha=0.8, scale=2.0, softcap=15.0), page=16, seed=12),
+        layer(att(heads=1, dim=24, rot_dim=2, vdim=40, kv_rank=24, base=7.0, scale=0.25), moe(8, 3, 24, (2, 1), 1.25))],
+        eps=1e-6, alpha=0.8, scale=2.0, softcap=12.0), page=16, seed=12),
 }
 
 

@@ -398,7 +398,7 @@ def test_the_router_with_sigmoid_scores_in_groups():
     from axon_amd.kernels import kernels
     k = kernels("float32")
     g = torch.Generator().manual_seed(5)
-    cases = [(6, 2, 3, 2, 2.5, 0.7), (16, 3, 2, 1, 1.5, 0.3), (64, 6, 8, 4, 1.0, 0.5), (256, 8, 8, 4, 2.0, 0.2), (5, 1, 1, 1, 0.5, 0.7),
+    cases = [(6, 2, 3, 2, 2.5, 0.7), (16, 3, 4, 2, 1.25, 0.3), (64, 6, 8, 4, 1.0, 0.5), (256, 8, 8, 4, 2.0, 0.2), (5, 1, 1, 1, 0.5, 0.7),
              (8, 2, 8, 3, 1.0, 0.7), (8, 8, 1, 1, 1.0, 0.0), (12, 4, 3, 1, 1.0, -3.0), (1000, 7, 10, 3, 1.0, 0.4), (70, 64, 1, 1, 1.0, 0.1)]
     for E, top, groups, keep, scale, spread in cases:
         T = 37
@@ -515,8 +515,8 @@ def test_the_norm_behind_the_sum_and_the_bent_logits(dtype):
     z = (torch.randn(5, 777, generator=g) * 40).cuda()
     wide = torch.zeros(5, 800, device="cuda")
     wide[:, :777] = z
-    k.softcap(wide[:, :777], 15.0)
-    assert float((wide[:, :777].cpu() - 15.0 * torch.tanh(z.cpu().double() / 15.0).float()).abs().max()) <= 1e-5
+    k.softcap(wide[:, :777], 11.0)
+    assert float((wide[:, :777].cpu() - 11.0 * torch.tanh(z.cpu().double() / 11.0).float()).abs().max()) <= 1e-5
     assert float(wide[:, 777:].abs().max()) == 0.0
 
 
@@ -528,7 +528,7 @@ def test_the_rotation_in_neighbouring_pairs_with_ramped_frequencies(dtype):
     from axon_amd.kernels import kernels
     k = kernels(dtype)
     g = torch.Generator().manual_seed(4)
-    for dim, rot_dim, dims, base, scaling in ((8, 4, 4, 100.0, (4.0, 16, 8.0, 1.0)), (32, 16, 16, 1e6, (8.0, 512, 32.0, 1.0)),
+    for dim, rot_dim, dims, base, scaling in ((8, 4, 4, 100.0, (4.0, 16, 8.0, 1.0)), (40, 16, 16, 5e5, (6.0, 256, 24.0, 1.0)),
                                               (8, 32, 16, 500.0, None), (16, 64, 64, 1e4, (2.0, 32, 4.0, 0.5)), (24, 2, 2, 7.0, None)):
         rot = {"base": base, "dims": dims}
         if scaling:

@@ -27,7 +27,7 @@ def random_config(rng):
         # a score's spread near 2.5 under the drawn weights, whatever the sizes
         scale = 2.5 / (2.25 * dim ** 0.5 + 1.5 * rot_dim ** 0.5)
         mixer = att(heads, dim, rot_dim, rng.choice([8, 16, 24, 48, 64]), rank, base=rng.choice([50.0, 10000.0, 1e6]), scale=scale,
-                    scaling=rng.choice([None, (4.0, 16, 8.0, 1.0), (8.0, 512, 32.0, 1.0), (2.0, 64, 4.0, 0.5)]))
+                    scaling=rng.choice([None, (4.0, 16, 8.0, 1.0), (6.0, 256, 24.0, 2.0), (2.0, 64, 4.0, 0.5)]))
         kind = rng.choice(["none", "dense", "moe", "moe"])
         if kind == "none":
             mlp = None
