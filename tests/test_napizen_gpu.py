@@ -241,6 +241,29 @@ def test_greedy_generation_through_the_entry_point(folders, name):
             assert float(row.max() - row[tok]) <= 0.1 * tolerance("bfloat16", logits)
 
 
+def test_the_command_line_generates_with_the_design(folders):
+    import os
+    import subprocess
+    import sys
+    from helpers import ROOT
+    name = "D"
+    cfg, W = P.load_plain(folders(name))
+    p, q = sequences(name, [9, 14], seed=9)
+    axon = [sys.executable, os.path.join(ROOT, "bin", "axon")]
+    ids = lambda seq: " ".join(map(str, seq))
+    r = subprocess.run(axon + ["gen", folders(name), ids(p), ids(q), "-n", "8", "--dtype", "float32", "--page-size", "64"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [[int(t) for t in line.split()] for line in r.stdout.splitlines()] == [
+        P.greedy_generate(cfg, W, p, 8), P.greedy_generate(cfg, W, q, 8)]
+    r = subprocess.run(axon + ["logits", folders(name), ids(p), "-k", "3", "--dtype", "float32"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr
+    top = torch.topk(P.forward_logits(cfg, W, p)[-1].float(), 3)
+    lines = [l.split() for l in r.stdout.splitlines() if "logit" in l]
+    assert [int(l[0]) for l in lines] == top.indices.tolist()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_the_trace_replay_program_runs_the_design(folders, plain_logits, tmp_path, dtype):
     name = "C"
