@@ -187,8 +187,9 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
   __shared__ __align__(16) bf16_t qs_all[LAM_WAVES][16 * QROW];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int groups = heads / 16;
-  const long item = (long)blockIdx.x * LAM_WAVES + wave;
-  const bool active = item < (long)n_tokens * groups;
+  // the step's last tokens first: they see the most positions, and the waves that start last should be the short ones
+  const long item = (long)n_tokens * groups - 1 - ((long)blockIdx.x * LAM_WAVES + wave);
+  const bool active = item >= 0;
   const int t = active ? (int)(item / groups) : 0, hg = active ? (int)(item % groups) : 0;
   const int width = rank + rot, qc = width / 32, rt = rank / 16;
   const int j = lane & 15, g = lane >> 4;
