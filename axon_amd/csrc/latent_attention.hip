@@ -174,7 +174,7 @@ __device__ inline la_bf16x8 la_frag(uint4 v) { return __builtin_bit_cast(la_bf16
 // lane) and the rounded weights, as they lie in the accumulators, as the second.  RT: tiles of 16
 // latent dims at most; QC: chunks of 32 key dims at most.  Pages hold a multiple of 64 positions.
 #define LAM_WAVES 2
-template <int RT, int QC>
+template <int RT, int QC, bool SINK>
 __global__ void __launch_bounds__(LAM_WAVES * 64)
 latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
@@ -187,9 +187,11 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
   __shared__ __align__(16) bf16_t qs_all[LAM_WAVES][16 * QROW];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int groups = heads / 16;
-  // the step's last tokens first: they see the most positions, and the waves that start last should be the short ones
-  const long item = (long)n_tokens * groups - 1 - ((long)blockIdx.x * LAM_WAVES + wave);
-  const bool active = item >= 0;
+  // without a window the step's last tokens first: they see the most positions, and the waves that start last
+  // should be the short ones; over a window most rows are equally long, and the tokens go in their order
+  const long n_items = (long)n_tokens * groups, at = (long)blockIdx.x * LAM_WAVES + wave;
+  const long item = window > 0 ? at : n_items - 1 - at;
+  const bool active = at < n_items;
   const int t = active ? (int)(item / groups) : 0, hg = active ? (int)(item % groups) : 0;
   const int width = rank + rot, qc = width / 32, rt = rank / 16;
   const int j = lane & 15, g = lane >> 4;
@@ -215,7 +217,7 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
 #pragma unroll
   for (int i = 0; i < RT; ++i) acc[i] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   // a sink is counted once a row: here when the wave walks all blocks, else by the kernel that folds them
-  const bool sunk = sink != nullptr && partial == nullptr;
+  const bool sunk = SINK && partial == nullptr;        // (an instance of its own: without a sink the running pair starts from constants)
   float m = sunk ? sink[hg * 16 + j] : -INFINITY, l = sunk ? 1.0f : 0.0f;
   // with `partial`: this wave takes one block of 64 positions (blockIdx.y after the token's first) and
   // leaves (o, m, l) unscaled for the kernel that folds a token's blocks in ascending order
@@ -360,9 +362,14 @@ static void launch_latent_mfma(const float* q_full, const void* cache, const int
                                hipStream_t stream) {
   const long items = (long)n_tokens * (heads / 16);
   dim3 grid((unsigned)((items + LAM_WAVES - 1) / LAM_WAVES), partial ? n_chunks : 1);
-  latent_attention_mfma_kernel<RT, QC><<<grid, LAM_WAVES * 64, 0, stream>>>(
-      q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
-      window, scale, sink, partial, n_chunks);
+  if (sink)
+    latent_attention_mfma_kernel<RT, QC, true><<<grid, LAM_WAVES * 64, 0, stream>>>(
+        q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
+        window, scale, sink, partial, n_chunks);
+  else
+    latent_attention_mfma_kernel<RT, QC, false><<<grid, LAM_WAVES * 64, 0, stream>>>(
+        q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
+        window, scale, sink, partial, n_chunks);
   if (partial)
     latent_attention_fold_kernel<<<n_tokens * heads, min(512, (rank + 63) / 64 * 64), 3 * n_chunks * sizeof(float), stream>>>(
         partial, o_lat, rank, n_chunks, sink, heads);
