@@ -321,6 +321,226 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
     if (dt < rt) *reinterpret_cast<float4*>(dst + 16 * dt) = make_float4(acc[dt][0] * inv, acc[dt][1] * inv, acc[dt][2] * inv, acc[dt][3] * inv);
 }
 
+// The same for steps of many tokens: four waves a block take four neighbouring tokens (and the same sixteen
+// heads).  Where these belong to one request (a prompt's portion) they read the same pages, and a block of
+// 64 positions is staged in LDS once for the four: its K rows [64][rank + rot] for the scores, then, in the
+// same buffer, its C^T rows [rank][64] for the weighted sums (rows 16 bytes longer than their content, as the
+// queries').  Each wave keeps its own mask, running pair and accumulators, and runs the chain of products
+// of the kernel above: the same bits.  Tokens of several requests in one block (decoding rows side by
+// side): every wave reads its own pages from memory, as above.
+#define LAS_WAVES 4
+#define LATENT_TOKENS_KERNEL_FROM 256           // (token, sixteen heads) items of a step from which four tokens share a block
+template <int RT, int QC, bool SHARED>
+__device__ __forceinline__ void latent_walk(const bf16_t* __restrict__ cache, const int32_t* __restrict__ pages, long page_elems,
+                                            int page_size, int width, int rank, int qc, int rt, int b_from, int b_to, bool active,
+                                            int lo, int pos, float scale, const bf16_t* qlane, bf16_t* stage, int j, int g,
+                                            float& m, float& l, la_f32x4 (&acc)[RT]) {
+  const int KROW = width + 8;
+  constexpr int VROW = 64 + 8;
+  for (int b = b_from; b <= b_to; ++b) {
+    const int p0 = b * 64, in0 = p0 % page_size;
+    const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
+    const bool mine = active && b >= lo / 64 && b <= pos / 64;
+    const bf16_t* kbase;
+    long krow_stride;
+    if constexpr (SHARED) {
+      __syncthreads();                               // the buffer's last readers are done
+      const uint4* src = reinterpret_cast<const uint4*>(page + (long)in0 * width);
+      const int per_row = width / 8, units = 64 * per_row;
+      {
+        // every load of the block's K rows in flight at once (the registers of the scores are free here)
+        uint4 held[QC];
+#pragma unroll
+        for (int e = 0; e < QC; ++e)
+          held[e] = src[min((int)threadIdx.x + e * LAS_WAVES * 64, units - 1)];
+#pragma unroll
+        for (int e = 0; e < QC; ++e) {
+          const int u = threadIdx.x + e * LAS_WAVES * 64;
+          if (u < units) *reinterpret_cast<uint4*>(stage + (u / per_row) * KROW + 8 * (u % per_row)) = held[e];
+        }
+      }
+      __syncthreads();
+      kbase = stage + 8 * g;
+      krow_stride = KROW;
+    } else {
+      kbase = page + (long)in0 * width + 8 * g;
+      krow_stride = width;
+    }
+    la_f32x4 s[4];
+    uint4 pf[2];
+    float fold = 1.0f;
+    if (mine) {
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt) {
+        s[pt] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        const bf16_t* krow = kbase + (long)(16 * pt + j) * krow_stride;
+        constexpr int QB = SHARED ? (QC < 4 ? QC : 4) : (QC < 10 ? QC : 10);
+#pragma unroll
+        for (int k0 = 0; k0 < QC; k0 += QB) {
+          uint4 kf[QB];
+#pragma unroll
+          for (int e = 0; e < QB; ++e)
+            if (k0 + e < qc) kf[e] = *reinterpret_cast<const uint4*>(krow + 32 * (k0 + e));
+#pragma unroll
+          for (int e = 0; e < QB; ++e)
+            if (k0 + e < qc) s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(kf[e]), la_frag(*reinterpret_cast<const uint4*>(qlane + 32 * (k0 + e))), s[pt], 0, 0, 0);
+        }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int p = p0 + 16 * pt + 4 * g + i;
+          const float v = (p >= lo && p <= pos) ? s[pt][i] * scale : -INFINITY;
+          s[pt][i] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      fold = expf(m - m_new);
+      float sum = 0.0f;
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float w = expf(s[pt][i] - m_new);        // 0 where the position is not seen
+          s[pt][i] = w;
+          sum += w;
+        }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l = fmaf(l, fold, sum);
+      m = m_new;
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+        pf[c] = make_uint4(pack2_bf16(s[2 * c][0], s[2 * c][1]), pack2_bf16(s[2 * c][2], s[2 * c][3]),
+                           pack2_bf16(s[2 * c + 1][0], s[2 * c + 1][1]), pack2_bf16(s[2 * c + 1][2], s[2 * c + 1][3]));
+    }
+    const bf16_t* vbase;
+    long vrow_stride;
+    if constexpr (SHARED) {
+      __syncthreads();                               // the K rows' readers are done
+      const bf16_t* src = page + (long)page_size * width + in0;
+      const int units = rank * 8;
+      {
+        constexpr int VU = (RT + 1) / 2;             // rank x 8 units of 16 bytes over 256 threads
+        uint4 held[VU];
+#pragma unroll
+        for (int e = 0; e < VU; ++e) {
+          const int u = min((int)threadIdx.x + e * LAS_WAVES * 64, units - 1);
+          held[e] = *reinterpret_cast<const uint4*>(src + (long)(u / 8) * page_size + 8 * (u % 8));
+        }
+#pragma unroll
+        for (int e = 0; e < VU; ++e) {
+          const int u = threadIdx.x + e * LAS_WAVES * 64;
+          if (u < units) *reinterpret_cast<uint4*>(stage + (u / 8) * VROW + 8 * (u % 8)) = held[e];
+        }
+      }
+      __syncthreads();
+      vbase = stage + 4 * g;
+      vrow_stride = VROW;
+    } else {
+      vbase = page + (long)page_size * width + in0 + 4 * g;
+      vrow_stride = page_size;
+    }
+    if (mine) {
+      constexpr int VB = SHARED ? 2 : 4;             // tiles of 16 dims whose rows are asked for together
+#pragma unroll
+      for (int d0 = 0; d0 < RT; d0 += VB) {
+        uint2 v[VB][4];
+#pragma unroll
+        for (int e = 0; e < VB; ++e) {
+          if (d0 + e < rt) {
+            const bf16_t* vrow = vbase + (long)(16 * (d0 + e) + j) * vrow_stride;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+              v[e][2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
+              v[e][2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+            }
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < VB; ++e) {
+          if (d0 + e < rt) {
+            acc[d0 + e] *= fold;
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+              acc[d0 + e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  la_frag(make_uint4(v[e][2 * c].x, v[e][2 * c].y, v[e][2 * c + 1].x, v[e][2 * c + 1].y)), la_frag(pf[c]), acc[d0 + e],
+                  0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int RT, int QC, bool SINK>
+__global__ void __launch_bounds__(LAS_WAVES * 64)
+latent_attention_mfma_tokens_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
+                                    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
+                                    const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
+                                    int rot, int page_size, int window, float scale, const float* __restrict__ sink) {
+  extern __shared__ __align__(16) bf16_t las_lds[];
+  bf16_t* stage = las_lds;                                                        // max(64 x (width + 8), rank x 72) elements
+  const int QROW = rank + rot + 8;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  bf16_t* qs = las_lds + max(64 * QROW, rank * 72) + wave * 16 * QROW;
+  const int groups = heads / 16;
+  const int n_tiles = (n_tokens + LAS_WAVES - 1) / LAS_WAVES;
+  // without a window the step's last tokens first (see the kernel above)
+  const int at = (int)blockIdx.x / groups, hg = (int)blockIdx.x % groups;
+  const int tile = window > 0 ? at : n_tiles - 1 - at;
+  const int t = tile * LAS_WAVES + wave;
+  const bool active = t < n_tokens;
+  const int width = rank + rot, qc = width / 32, rt = rank / 16;
+  const int j = lane & 15, g = lane >> 4;
+  if (active) {
+    const int per_row = width / 8;
+    for (int idx = lane; idx < 16 * per_row; idx += 64) {
+      const int row = idx / per_row, part = idx % per_row;
+      const float* src = q_full + ((long)t * heads + hg * 16 + row) * width + 8 * part;
+      const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+      *reinterpret_cast<uint4*>(qs + row * QROW + 8 * part) =
+          make_uint4(pack2_bf16(a.x, a.y), pack2_bf16(a.z, a.w), pack2_bf16(b.x, b.y), pack2_bf16(b.z, b.w));
+    }
+  }
+  // the block's tokens: one request (its pages staged once for all) or several (every wave on its own)
+  const int t_first = tile * LAS_WAVES, t_last = min(t_first + LAS_WAVES, n_tokens) - 1;
+  bool same = true;
+  int b_from = 1 << 30, b_to = -1;
+  for (int u = t_first; u <= t_last; ++u) {
+    same = same && seq_rows[u] == seq_rows[t_first];
+    const int p = positions[u];
+    b_from = min(b_from, (window > 0 ? max(0, p + 1 - window) : 0) / 64);
+    b_to = max(b_to, p / 64);
+  }
+  const bf16_t* qlane = qs + j * QROW + 8 * g;
+  const int pos = active ? positions[t] : 0;
+  const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int32_t* pages = block_table + (long)seq_rows[active ? t : t_first] * table_stride;
+  const long page_elems = (long)page_size * (width + rank);
+  la_f32x4 acc[RT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i) acc[i] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float m = (SINK && active) ? sink[hg * 16 + j] : -INFINITY, l = SINK ? 1.0f : 0.0f;
+  __syncthreads();
+  if (same)
+    latent_walk<RT, QC, true>(cache, pages, page_elems, page_size, width, rank, qc, rt, b_from, b_to, active, lo, pos, scale, qlane, stage,
+                              j, g, m, l, acc);
+  else if (active)
+    latent_walk<RT, QC, false>(cache, pages, page_elems, page_size, width, rank, qc, rt, lo / 64, pos / 64, true, lo, pos, scale, qlane,
+                               stage, j, g, m, l, acc);
+  if (!active) return;
+  const float inv = 1.0f / l;
+  float* dst = o_lat + ((long)t * heads + hg * 16 + j) * rank + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < RT; ++dt)
+    if (dt < rt) *reinterpret_cast<float4*>(dst + 16 * dt) = make_float4(acc[dt][0] * inv, acc[dt][1] * inv, acc[dt][2] * inv, acc[dt][3] * inv);
+}
+
 // o_lat[row, :] = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) l_c over a row's blocks in ascending order
 // (M the largest m_c; a block that saw nothing has l = 0 and weighs nothing).  One block per (token,
 // head): the blocks' (m, l) once into LDS, all loads in flight together, their weights from there, then
@@ -353,6 +573,43 @@ latent_attention_fold_kernel(const float* __restrict__ partial, float* __restric
     for (int c = 0; c < n_chunks; ++c) o = fmaf(weight[c], src[(long)c * (rank + 2) + d], o);
     o_lat[(long)blockIdx.x * rank + d] = o * inv;
   }
+}
+
+// Steps of many tokens (no blocks side by side): four tokens a block, their pages staged in LDS once.
+static long latent_tokens_lds(int rank, int rot) {
+  const long qrow = rank + rot + 8, stage = 64 * qrow > (long)rank * 72 ? 64 * qrow : (long)rank * 72;
+  return (stage + LAS_WAVES * 16 * qrow) * (long)sizeof(bf16_t);
+}
+#define LATENT_LDS_MOST (160 * 1024)
+
+template <int RT, int QC>
+static int launch_latent_mfma_tokens(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
+                                     const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
+                                     int rot, int page_size, int window, float scale, const float* sink, hipStream_t stream) {
+  const int lds = (int)latent_tokens_lds(rank, rot);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_mfma_tokens_kernel<RT, QC, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LATENT_LDS_MOST);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_mfma_tokens_kernel<RT, QC, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, LATENT_LDS_MOST);
+    if (e != hipSuccess) {
+      axk_set_error("latent_attention: cannot reserve %d bytes of LDS: %s", LATENT_LDS_MOST, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  const unsigned grid = (unsigned)(((n_tokens + LAS_WAVES - 1) / LAS_WAVES) * (heads / 16));
+  if (sink)
+    latent_attention_mfma_tokens_kernel<RT, QC, true><<<grid, LAS_WAVES * 64, lds, stream>>>(
+        q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size, window,
+        scale, sink);
+  else
+    latent_attention_mfma_tokens_kernel<RT, QC, false><<<grid, LAS_WAVES * 64, lds, stream>>>(
+        q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size, window,
+        scale, sink);
+  return 0;
 }
 
 template <int RT, int QC>
@@ -455,6 +712,21 @@ extern "C" int axk_latent_attention(const float* q_full, const void* cache, cons
                 partial_floats, need);
     if (need == 0) partial = nullptr;
     const int n_chunks = latent_blocks_side_by_side(window, span);
+    if (partial == nullptr && (long)n_tokens * (heads / 16) >= LATENT_TOKENS_KERNEL_FROM && latent_tokens_lds(rank, rot) <= LATENT_LDS_MOST) {
+      int rc;
+      if (rank <= 64 && rank + rot <= 128)
+        rc = launch_latent_mfma_tokens<4, 4>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank,
+                                             rot, page_size, window, scale, sink, s);
+      else if (rank <= 128 && rank + rot <= 256)
+        rc = launch_latent_mfma_tokens<8, 8>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank,
+                                             rot, page_size, window, scale, sink, s);
+      else
+        rc = launch_latent_mfma_tokens<32, 20>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads,
+                                               rank, rot, page_size, window, scale, sink, s);
+      if (rc) return rc;
+      AXK_LAUNCH_CHECK("latent_attention");
+      return 0;
+    }
     if (rank <= 64 && rank + rot <= 128)
       launch_latent_mfma<4, 4>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
                                page_size, window, scale, sink, partial, n_chunks, s);

@@ -207,6 +207,22 @@ def test_unequal_requests_side_by_side_with_pages_and_slots_used_again(folders, 
         assert float((alone[2] - got[2]).abs().max()) <= 2 * tolerance(dtype, plain_logits(name, seqs[2]))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_portions_of_several_requests_in_one_step(folders, plain_logits, name, dtype):
+    """Hundreds of tokens a step with heads in sixteens: the attention takes four neighbouring tokens a block
+    and stages their pages once where they are one request's; blocks that hold the end of one request and
+    the start of the next, or decoded rows of several, let every token read its own pages."""
+    lengths = [150, 131, 97, 64]
+    seqs = dict(enumerate(sequences(name, lengths, seed=11)))
+    eng = engine_for(folders(name), dtype, 64, 9, max_seqs=4, max_seq_len=192, max_batch_tokens=512, shuffle_pages_seed=3)
+    sched = [[(0, 101), (1, 99), (2, 95), (3, 1)], [(0, 47), (1, 30), (2, 1), (3, 62)], [(0, 2), (1, 2), (2, 1), (3, 1)]]
+    got, chose = run_schedule(eng, name, seqs, sched)
+    for r in seqs:
+        assert_close(got[r], plain_logits(name, seqs[r], dtype, chose[r]), dtype, f"request {r}")
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("name", ["A", "D"])
 def test_long_decoding_across_many_pages(folders, plain_logits, name):
     n = 250
