@@ -211,6 +211,10 @@ int axk_layernorm(const float* x, const int32_t* rows, const void* gain, int gai
                   float eps, void* stream);
 // v[r, i] = cap tanh(v[r, i] / cap), in place on float32 rows row_stride apart.
 int axk_softcap(float* v, long row_stride, int n_rows, int n, float cap, void* stream);
+// v[r, i] *= factor, in place on float32 rows row_stride apart.
+int axk_scale_rows(float* v, long row_stride, int n_rows, int n, float factor, void* stream);
+// x[i] += factor * y[i] on n float32 values.
+int axk_add_scaled(float* x, const float* y, float factor, long n, void* stream);
 // out[i] = x[i] in the compute dtype.
 int axk_round_rows(const float* x, void* out, long n, void* stream);
 // out[t, :] = [a[t, :] | b[t, :]] in the compute dtype (a [n_rows, wa], b [n_rows, wb] float32).
@@ -231,12 +235,15 @@ int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, flo
 // sigmoid(alpha g) (u + shift); an infinite limit, alpha 1 and shift 0 are silu(gate) up.  gate (float32,
 // rows gate_row_stride apart): out is multiplied by sigmoid(gate[orow, g ogs + n]), or with
 // gate_per_group by sigmoid(gate[orow, g]), one number a group.  Strides count elements.  An output's chain over k depends on
-// k, the strides' alignment and the build alone (axk_grouped_gemm_uses_mfma says which chain).
+// k, the strides' alignment and the build alone (axk_grouped_gemm_uses_mfma says which chain).  row_scale (float32
+// [out rows], or null): the sums of out row r are multiplied by row_scale[r] before bias and epilogue (a factor on
+// the row of X).
 int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride, long x_group_stride);
 int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
                      const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32, long out_row_stride,
                      long out_group_stride, const int32_t* out_rows, const float* gate, long gate_row_stride,
-                     int gate_per_group, int glu, float glu_limit, float glu_alpha, float glu_shift, const int32_t* tiles,
+                     int gate_per_group, const float* row_scale, int glu, float glu_limit, float glu_alpha, float glu_shift,
+                     const int32_t* tiles,
                      const int32_t* n_tiles, int max_tiles,
                      int tile_rows, int m, int n, int k, int groups, void* stream);
 
@@ -245,22 +252,24 @@ int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_grou
 // axk_route_scored: scores s = sigmoid(logits) that do not compete; chosen by s + correction (float32
 // [n_experts], or null) among the experts of the `keep` best of `groups` equal groups of neighbours (a
 // group's score: the sum of its two largest choice scores), weights s / (sum of the chosen s + 1e-20)
-// * scale.  Up to 1,024 experts in up to 64 groups, up to 64 a token.
+// * scale (without `normalize`: s * scale); rows of logits are logits_stride apart.  Up to 1,024 experts in up to
+// 64 groups, up to 64 a token.
 // axk_route_sort: the pairs p = t top + k in expert order (sorted, and each one's token in
 // sorted_tokens) and the tiles (of up to tile_rows rows) of the grouped product, at most
 // axk_route_max_tiles of them.
 // place_of [n_pairs] (or null): where each pair stands in `sorted`; first_of [n_experts + 1] (or
 // null): where each expert's pairs start there.
 // axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending (with
-// place_of: rows[place_of[t top + k], :]).  axk_gather_rows: out[r, :] = x[rows[r], :] (elem).
+// place_of: rows[place_of[t top + k], :]); weights may be null (all 1); extra (float32 [n_tokens, width], or null) is
+// a further row a token, times sigmoid(extra_gate[t extra_gate_stride]) if extra_gate is given.  axk_gather_rows: out[r, :] = x[rows[r], :] (elem).
 int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights, void* stream);
-int axk_route_scored(const float* logits, const float* correction, int n_tokens, int n_experts, int top, int groups, int keep,
-                     float scale, int32_t* experts, float* weights, void* stream);
+int axk_route_scored(const float* logits, long logits_stride, const float* correction, int n_tokens, int n_experts, int top,
+                     int groups, int keep, float scale, int normalize, int32_t* experts, float* weights, void* stream);
 int axk_route_max_tiles(int n_pairs, int n_experts, int tile_rows);
 int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted, int32_t* sorted_tokens,
                    int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of, int tile_rows, void* stream);
 int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width, int accumulate,
-                      const int32_t* place_of, void* stream);
+                      const int32_t* place_of, const float* extra, const float* extra_gate, long extra_gate_stride, void* stream);
 int axk_gather_rows(const void* x, long x_stride, const int32_t* rows, void* out, int n_rows, int width, void* stream);
 
 // A short causal convolution per channel and a gated linear recurrence (csrc/recurrent.hip).  A
@@ -285,6 +294,28 @@ int axk_gated_scan(const float* gates, const float* u, const void* y, long y_str
                    const void* lam, int lam_is_f32, float decay, float* state, long state_stride, const int32_t* spans,
                    int n_spans, const int32_t* positions, const int32_t* seq_rows, void* out, int channels, int block_width,
                    int taps, float* terms, int n_tokens, void* stream);
+
+// A selective state-space mixer in its recurrent form (csrc/state_space.hip).  A request's state row (float32, rows
+// state_stride apart) holds two copies of copy_elems floats: the heads' states [heads][N][P] first, and from tail_at
+// [taps - 1][channels] of the convolution's last inputs, oldest first; the state behind position p is in copy p & 1.
+// axk_state_conv: u[t, c] = act(bias[c] + sum_k w[c, k] in(t - (taps - 1 - k))) over float32 rows x (silu: act is
+// silu, else none), inputs before the step from the state; with heads > 0 also terms[t, h] = (dt, a) with
+// dt = softplus(raw[t, h] + dt_bias[h]), a = exp(-exp(a_log[h]) dt).  Reads the state only.
+// axk_state_space_scan: per request of the step (spans [n][3] = (slot, first token, tokens); null: each token a
+// request of its own in slot seq_rows[t]) and head, over its tokens in order, S = a S + dt B x^T, y = S^T C + D x
+// with u [T, channels] = [x: heads P | B: groups N | C: groups N]; y float32 [T, heads P]; then the state row is
+// brought up to date (S, and the convolution's inputs from conv_in, float32 rows conv_in_stride apart).
+// axk_gated_group_norm: out[t] = rms in `parts` equal parts of (y[t] silu(z[t])), times gain; out elem [T, width].
+int axk_state_conv(const float* x, long x_stride, const void* w, const void* bias, int bias_is_f32, int silu, const float* state,
+                   long state_stride, long copy_elems, long tail_at, const int32_t* positions, const int32_t* seq_rows, float* u,
+                   int n_tokens, int channels, int taps, const float* raw, long raw_stride, const void* dt_bias,
+                   int dt_bias_is_f32, const void* a_log, int a_log_is_f32, float* terms, int heads, void* stream);
+int axk_state_space_scan(const float* u, const float* terms, const void* d_skip, int d_is_f32, float* state, long state_stride,
+                         long copy_elems, long tail_at, const int32_t* spans, int n_spans, const int32_t* positions,
+                         const int32_t* seq_rows, const float* conv_in, long conv_in_stride, float* y, int heads, int groups,
+                         int vdim, int n_state, int taps, void* stream);
+int axk_gated_group_norm(const float* y, const float* z, long z_stride, const void* gain, int gain_is_f32, float eps, void* out,
+                         int n_tokens, int width, int parts, void* stream);
 
 // Attention over a latent cache (csrc/latent_attention.hip); a page is [page_size][rank + rot] elem
 // (the latent and the rotated key part of each position), then [rank][page_size] (the latents again,
@@ -321,16 +352,18 @@ int axk_latent_attention(const float* q_full, const void* cache, const int32_t* 
 // each, v_width values; v_at may equal k_at), units RMS-normed with a gain shared by all units (null: no
 // norm), the first `rot` dims rotated by table [T, rot / 2, 2] (sin, cos; both scaled by `magnitude`) in
 // pairs (2i, 2i + 1) if `neighbours` else (i, i + rot / 2); queries into q_out elem [T, n_q dim], keys and
-// values into the page (if write_kv).
+// values into the page (if write_kv).  q_temp_every > 0: a query at position p is multiplied by
+// 1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1).
 int axk_heads_prepare(const float* proj, long stride, int q_at, int n_q, int k_at, int n_k, int v_at, int v_width, int dim,
                       const void* q_gain, int q_gain_is_f32, const void* k_gain, int k_gain_is_f32, float eps, int rot,
                       int neighbours, float magnitude, const float* table, const int32_t* positions, const int32_t* seq_rows,
                       const int32_t* block_table, int table_stride, void* cache, int page_size, void* q_out, int n_tokens,
-                      int write_kv, void* stream);
+                      int write_kv, float q_temp_coef, int q_temp_every, void* stream);
 // axk_masked_attention: q elem [T, heads maps dim] -> out elem [T, heads vdim].  mask_kind 0: all earlier
 // positions; 1: the last mask_size positions; 2: the earlier positions of the same chunk of mask_size.
 // softcap > 0: s <- softcap tanh(s / softcap).  maps 2: o = rms(a_1 - lambda a_2, eps) out_scale.  gate
-// (float32 rows of gate_stride, or null): o *= sigmoid(gate).  tiles (int32 [n_tiles, 2]: first token,
+// (float32 rows of gate_stride, or null): o *= sigmoid(gate), heads vdim numbers a row, or with gate_per_head
+// one a head.  sink > -inf: the softmax's sum also holds exp(sink), a key of that score without a value.  tiles (int32 [n_tiles, 2]: first token,
 // count; up to 16 consecutive tokens of one request each) or null (every token a tile of its own) are
 // what the matrix-core kernel works on where axk_masked_attention_uses_mfma says 1.
 // partial: axk_masked_attention_workspace floats (steps of few tokens under a window or in chunks: the
@@ -342,7 +375,8 @@ int axk_masked_attention(const void* q, const void* cache, const int32_t* block_
                          const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
                          int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size, int mask_kind,
                          int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
-                         const int32_t* tiles, int n_tiles, float* partial, long partial_floats, void* stream);
+                         const int32_t* tiles, int n_tiles, float* partial, long partial_floats, float sink, int gate_per_head,
+                         void* stream);
 
 #ifdef __cplusplus
 }

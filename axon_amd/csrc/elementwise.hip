@@ -399,6 +399,33 @@ extern "C" int axk_softcap(float* v, long row_stride, int n_rows, int n, float c
   return 0;
 }
 
+// v[r, i] *= factor, in place on float32 rows.
+__global__ void scale_rows_kernel(float* __restrict__ v, long row_stride, int n, float factor) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) v[(long)blockIdx.y * row_stride + i] *= factor;
+}
+
+extern "C" int axk_scale_rows(float* v, long row_stride, int n_rows, int n, float factor, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n_rows <= 65535 && n > 0, "scale_rows: bad sizes rows=%d n=%d", n_rows, n);
+  if (n_rows == 0) return 0;
+  scale_rows_kernel<<<dim3(ceil_div(n, 256), n_rows), 256, 0, (hipStream_t)stream>>>(v, row_stride, n, factor);
+  AXK_LAUNCH_CHECK("scale_rows");
+  return 0;
+}
+
+// x[i] += factor * y[i] on float32 values (the product is rounded before the sum).
+__global__ void add_scaled_kernel(float* __restrict__ x, const float* __restrict__ y, float factor, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = __fadd_rn(x[i], __fmul_rn(factor, y[i]));
+}
+
+extern "C" int axk_add_scaled(float* x, const float* y, float factor, long n, void* stream) {
+  if (n <= 0) return 0;
+  add_scaled_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, y, factor, n);
+  AXK_LAUNCH_CHECK("add_scaled");
+  return 0;
+}
+
 // out[i] = x[i] in the compute dtype.
 __global__ void round_rows_kernel(const float* __restrict__ x, elem_t* __restrict__ out, long n) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -14,7 +14,8 @@
 // Epilogues: bias; a gated linear unit with clamps (W holds 2 N rows a group, gate rows then up
 // rows: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + shift); an
 // infinite limit, alpha 1 and shift 0 give silu(gate) up); a multiplication by sigmoid(gate[orow, g ogs + n]),
-// or by sigmoid(gate[orow, g]), one number a group; out in float32 or in the compute dtype.
+// or by sigmoid(gate[orow, g]), one number a group; a factor a row on X (row_scale[orow], float32: the sums are
+// multiplied by it before bias and unit, as if the row of X had been); out in float32 or in the compute dtype.
 //
 // The K-reduction of one output is one chain in ascending k that depends on K and the build alone
 // (32-bit FMA, or 16x16x32 MFMAs where the bfloat16 build can use them: K a multiple of 32 and
@@ -30,6 +31,7 @@ struct GroupedArgs {
   const elem_t* w; const void* bias; int bias_is_f32;
   void* out; int out_is_f32; long out_row_stride; long out_group_stride; const int32_t* out_rows;
   const float* gate; long gate_row_stride; int gate_per_group;
+  const float* row_scale;
   int glu; float glu_limit; float glu_alpha; float glu_shift;
   const int32_t* tiles; const int32_t* n_tiles;
   int M, N, K, G;
@@ -50,6 +52,11 @@ __device__ inline float clamped_glu(float gate, float up, float limit, float alp
 }
 
 __device__ inline void gg_store(const GroupedArgs& a, int g, int orow, int n, float v, float up) {
+  if (a.row_scale) {                    // the row of X counts row_scale[orow] times: the product is linear in it
+    const float w = a.row_scale[orow];
+    v *= w;
+    up *= w;
+  }
   if (a.bias) {
     const int per = a.glu ? 2 * a.N : a.N;
     v += load_vec(a.bias, a.bias_is_f32, g * per + n);
@@ -314,8 +321,8 @@ extern "C" int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride
 extern "C" int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
                                 const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32,
                                 long out_row_stride, long out_group_stride, const int32_t* out_rows, const float* gate,
-                                long gate_row_stride, int gate_per_group, int glu, float glu_limit, float glu_alpha,
-                                float glu_shift, const int32_t* tiles,
+                                long gate_row_stride, int gate_per_group, const float* row_scale, int glu, float glu_limit,
+                                float glu_alpha, float glu_shift, const int32_t* tiles,
                                 const int32_t* n_tiles, int max_tiles, int tile_rows, int m, int n, int k, int groups,
                                 void* stream) {
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0 && groups > 0, "grouped_gemm: bad sizes M=%d N=%d K=%d groups=%d", m, n, k, groups);
@@ -328,8 +335,8 @@ extern "C" int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, 
   if (row_tiles == 0) return 0;
   AXK_REQUIRE(groups <= 65535 && ceil_div(n, GG_COLS) <= 65535, "grouped_gemm: %d groups of %d columns are too many", groups, n);
   GroupedArgs a{x, x_is_f32, x_row_stride, x_group_stride, x_rows, (const elem_t*)w, bias, bias_is_f32, out, out_is_f32,
-                out_row_stride, out_group_stride, out_rows, gate, gate_row_stride, gate_per_group, glu, glu_limit, glu_alpha, glu_shift,
-                tiles, n_tiles,
+                out_row_stride, out_group_stride, out_rows, gate, gate_row_stride, gate_per_group, row_scale, glu, glu_limit, glu_alpha,
+                glu_shift, tiles, n_tiles,
                 m, n, k, groups};
   dim3 grid(row_tiles, ceil_div(n, GG_COLS), tiles ? 1 : groups);
   hipStream_t s = (hipStream_t)stream;

@@ -6,7 +6,9 @@
 //   * what a position sees: every earlier position, the last `size` positions (a sliding window), or
 //     the earlier positions of its own chunk of `size` (chunks counted from position 0);
 //   * scores bent by cap tanh(s / cap);
-//   * an elementwise gate sigmoid(g) on the concatenated heads.
+//   * a sink in the softmax: a key of a given score that has no value (its weight only enters the sum);
+//   * a query temperature by position, q (1 + coef ln(floor((p + 1) / every) + 1));
+//   * a gate sigmoid(g) on the concatenated heads, a number an element or a number a head.
 //
 // A page of the cache holds, for its positions, the key rows [page_size][kv_heads maps dim] and behind
 // them the values with the positions of one dim side by side, [kv_heads vdim][page_size] (the operand
@@ -37,8 +39,10 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
                      int k_gain_is_f32, float eps, int rot, int neighbours, float magnitude, const float* __restrict__ table,
                      const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                      const int32_t* __restrict__ block_table, int table_stride, elem_t* __restrict__ cache, int page_size,
-                     elem_t* __restrict__ q_out, int write_kv) {
+                     elem_t* __restrict__ q_out, int write_kv, float q_temp_coef, int q_temp_every) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // a query's temperature by its position: 1 + coef ln(floor((p + 1) / every) + 1), or 1
+  const float q_temp = q_temp_every > 0 ? 1.0f + q_temp_coef * logf((float)((positions[t] + 1) / q_temp_every + 1)) : 1.0f;
   const float* row = proj + (long)t * stride;
   const int half = rot / 2;
   const float* tab = table + (long)t * half * 2;
@@ -58,6 +62,7 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
     elem_t* dst = is_q ? q_out + ((long)t * n_q + u) * dim : page_base + (long)in_page * kw + (long)(u - n_q) * dim;
     const void* gain = is_q ? q_gain : k_gain;
     const int gain_is_f32 = is_q ? q_gain_is_f32 : k_gain_is_f32;
+    const float temp = is_q ? q_temp : 1.0f;
     float inv = 1.0f;
     if (gain != nullptr) {
       float ss = 0.0f;
@@ -72,13 +77,13 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
         b = (b * inv) * load_vec(gain, gain_is_f32, ib);
       }
       const float s = tab[2 * i] * magnitude, c = tab[2 * i + 1] * magnitude;
-      dst[ia] = from_float(__fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s)));
-      dst[ib] = from_float(__fadd_rn(__fmul_rn(b, c), __fmul_rn(a, s)));
+      dst[ia] = from_float(__fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s)) * temp);
+      dst[ib] = from_float(__fadd_rn(__fmul_rn(b, c), __fmul_rn(a, s)) * temp);
     }
     for (int i = rot + lane; i < dim; i += 64) {
       float a = src[i];
       if (gain != nullptr) a = (a * inv) * load_vec(gain, gain_is_f32, i);
-      dst[i] = from_float(a);
+      dst[i] = from_float(a * temp);
     }
   }
   if (!write_kv) return;
@@ -98,7 +103,7 @@ masked_attention_kernel(const elem_t* __restrict__ q, const elem_t* __restrict__
                         int table_stride, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                         const float* __restrict__ gate, long gate_stride, elem_t* __restrict__ out, int n_tokens, int heads,
                         int kv_heads, int maps, int dim, int vdim, int page_size, int mask_kind, int mask_size, float scale,
-                        float softcap, float lambda, float out_scale, float eps) {
+                        float softcap, float lambda, float out_scale, float eps, float sink, int gate_per_head) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long item = (long)blockIdx.x * MA_WAVES + wave;
@@ -157,6 +162,7 @@ masked_attention_kernel(const elem_t* __restrict__ q, const elem_t* __restrict__
         }
       }
     }
+    if (sink > -INFINITY) l += expf(sink - m);       // a key of this score that has no value
     const float inv = 1.0f / l;
 #pragma unroll
     for (int i = 0; i < MA_OWN; ++i) o[i] = mp == 0 ? acc[i] * inv : o[i] - lambda * (acc[i] * inv);
@@ -175,7 +181,7 @@ masked_attention_kernel(const elem_t* __restrict__ q, const elem_t* __restrict__
     const int d = lane + 64 * i;
     if (d >= vdim) continue;
     float v = o[i];
-    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(long)t * gate_stride + (long)h * vdim + d]));
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(long)t * gate_stride + (gate_per_head ? (long)h : (long)h * vdim + d)]));
     dst[d] = from_float(v);
   }
 }
@@ -351,7 +357,12 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, PTR kbase, int kstride, P
 template <int MAPS, int DT>
 __device__ inline void ma_finish(MaState<MAPS, DT>& st, bool my_col, int my_tok, int my_head, int heads, int vdim, int dt_n,
                                  const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out, float lambda,
-                                 float out_scale, float eps, int g) {
+                                 float out_scale, float eps, int g, float sink_log2, int gate_per_head) {
+  // the sink: a key of that score (in units of log2 e, like the running maxima) that has no value
+  if (sink_log2 > -INFINITY) {
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) st.l[mp] += __builtin_amdgcn_exp2f(sink_log2 - st.m[mp]);
+  }
   const float inv0 = 1.0f / st.l[0];
   float ss = 0.0f;
 #pragma unroll
@@ -375,7 +386,8 @@ __device__ inline void ma_finish(MaState<MAPS, DT>& st, bool my_col, int my_tok,
   }
   if (!my_col) return;
   bf16_t* dst = out + ((long)my_tok * heads + my_head) * vdim + 4 * g;
-  const float* gsrc = gate ? gate + (long)my_tok * gate_stride + (long)my_head * vdim + 4 * g : nullptr;
+  const float* gsrc = gate && !gate_per_head ? gate + (long)my_tok * gate_stride + (long)my_head * vdim + 4 * g : nullptr;
+  const float head_gate = gate && gate_per_head ? 1.0f / (1.0f + expf(-gate[(long)my_tok * gate_stride + my_head])) : 1.0f;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
     if (dt < dt_n) {
@@ -385,6 +397,7 @@ __device__ inline void ma_finish(MaState<MAPS, DT>& st, bool my_col, int my_tok,
         o[i] = st.acc[0][dt][i];
         if (MAPS == 2) o[i] = (o[i] * norm) * out_scale;
         if (gsrc) o[i] *= 1.0f / (1.0f + expf(-gsrc[16 * dt + i]));
+        o[i] *= head_gate;
       }
       *reinterpret_cast<uint2*>(dst + 16 * dt) = make_uint2(pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]));
     }
@@ -401,7 +414,7 @@ masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
                              const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out,
                              const int32_t* __restrict__ tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
                              int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
-                             float* __restrict__ partial, int n_chunks) {
+                             float* __restrict__ partial, int n_chunks, float sink_log2, int gate_per_head) {
   constexpr int QMAP = KC * 32, QROW = MAPS * QMAP + 8;      // rows 16 bytes longer than their chunks: 16 rows, 16 banks apart
   __shared__ __align__(16) bf16_t qs[16 * QROW];
   const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
@@ -473,7 +486,8 @@ masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     }
     return;
   }
-  ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g);
+  ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g, sink_log2,
+                      gate_per_head);
 }
 
 // The blocks of a single token's (head, map) folded in ascending order, a_mp = sum_c e^(m_c - M) o_c /
@@ -484,7 +498,7 @@ template <int MAPS>
 __global__ void __launch_bounds__(64)
 masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, const int32_t* __restrict__ tiles,
                              const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out, int heads, int vdim,
-                             float lambda, float out_scale, float eps) {
+                             float lambda, float out_scale, float eps, float sink_log2, int gate_per_head) {
   const int t = tiles ? tiles[2 * blockIdx.x] : (int)blockIdx.x, n = tiles ? tiles[2 * blockIdx.x + 1] : 1;
   if (n != 1) return;
   const int h = blockIdx.y, lane = threadIdx.x;
@@ -527,6 +541,7 @@ masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, co
         }
       }
     }
+    if (sink_log2 > -INFINITY) L += exp2f(sink_log2 - M);
     const float inv = 1.0f / L;
 #pragma unroll
     for (int i = 0; i < MA_OWN; ++i) {
@@ -548,7 +563,7 @@ masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, co
     const int d = lane + 64 * i;
     if (d >= vdim) continue;
     float v = o[i];
-    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(long)t * gate_stride + (long)h * vdim + d]));
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(long)t * gate_stride + (gate_per_head ? (long)h : (long)h * vdim + d)]));
     dst[d] = from_float(v);
   }
 }
@@ -566,7 +581,7 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
                                const int32_t* __restrict__ seq_rows, const float* __restrict__ gate, long gate_stride,
                                bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int heads, int kv_heads, int dim,
                                int vdim, int page_size, int mask_kind, int mask_size, float scale, float softcap, float lambda,
-                               float out_scale, float eps) {
+                               float out_scale, float eps, float sink_log2, int gate_per_head) {
   extern __shared__ __align__(16) bf16_t stage[];       // keys [64][MAPS dim + 8], then values [vdim][64 + 8]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
   const int grp = heads / kv_heads, hb_n = (grp + MAS_WAVES - 1) / MAS_WAVES;
@@ -658,7 +673,8 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
                              ncols == 16 && p0 >= lo_last && p0 + 63 <= pos_first, dim, dt_n, scale, softcap, j, g);
   }
   if (active)
-    ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g);
+    ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g, sink_log2,
+                      gate_per_head);
 }
 
 // Blocks of positions a single token can touch under its mask (0: no bound).
@@ -671,7 +687,7 @@ static int launch_masked_mfma(const void* q, const void* cache, const int32_t* b
                               const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
                               const int32_t* tiles, int n_tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
                               int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
-                              float* partial, hipStream_t stream) {
+                              float* partial, float sink_log2, int gate_per_head, hipStream_t stream) {
   const int grp = heads / kv_heads;
   const size_t lds = ((size_t)64 * (MAPS * dim + 8) + (size_t)vdim * (64 + 8)) * sizeof(bf16_t);
   if (tiles != nullptr && partial == nullptr && KC <= 4 && DT <= 8 && lds <= 64 * 1024) {
@@ -688,16 +704,19 @@ static int launch_masked_mfma(const void* q, const void* cache, const int32_t* b
     masked_attention_staged_kernel<MAPS, DT, KC>
         <<<dim3(n_tiles, kv_heads * ((grp + MAS_WAVES - 1) / MAS_WAVES)), MAS_WAVES * 64, lds, stream>>>(
             (const bf16_t*)q, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride,
-            (bf16_t*)out, tiles, heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps);
+            (bf16_t*)out, tiles, heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps,
+            sink_log2, gate_per_head);
     return 0;
   }
   const int n_chunks = partial ? masked_chunks(mask_kind, mask_size) : 1;
   masked_attention_mfma_kernel<MAPS, DT, KC><<<dim3(n_tiles, heads, n_chunks), 64, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, (bf16_t*)out, tiles,
-      heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps, partial, n_chunks);
+      heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps, partial, n_chunks,
+      sink_log2, gate_per_head);
   if (partial)
     masked_attention_fold_kernel<MAPS><<<dim3(n_tiles, heads), 64, 0, stream>>>(partial, n_chunks, tiles, gate, gate_stride,
-                                                                              (bf16_t*)out, heads, vdim, lambda, out_scale, eps);
+                                                                              (bf16_t*)out, heads, vdim, lambda, out_scale, eps,
+                                                                              sink_log2, gate_per_head);
   return 0;
 }
 #endif
@@ -708,7 +727,7 @@ extern "C" int axk_heads_prepare(const float* proj, long stride, int q_at, int n
                                  int dim, const void* q_gain, int q_gain_is_f32, const void* k_gain, int k_gain_is_f32, float eps,
                                  int rot, int neighbours, float magnitude, const float* table, const int32_t* positions,
                                  const int32_t* seq_rows, const int32_t* block_table, int table_stride, void* cache, int page_size,
-                                 void* q_out, int n_tokens, int write_kv, void* stream) {
+                                 void* q_out, int n_tokens, int write_kv, float q_temp_coef, int q_temp_every, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && n_q > 0 && n_k > 0 && dim > 0 && v_width > 0 && page_size > 0,
               "heads_prepare: bad sizes T=%d q units=%d k units=%d dim=%d values=%d page=%d", n_tokens, n_q, n_k, dim, v_width,
               page_size);
@@ -720,7 +739,8 @@ extern "C" int axk_heads_prepare(const float* proj, long stride, int q_at, int n
   const int per_token = n_tokens >= 1024 ? 1 : min((n_q + n_k + 3) / 4, 16);
   heads_prepare_kernel<<<dim3(n_tokens, per_token), 256, 0, (hipStream_t)stream>>>(
       proj, stride, q_at, n_q, k_at, n_k, v_at, v_width, dim, q_gain, q_gain_is_f32, k_gain, k_gain_is_f32, eps, rot, neighbours,
-      magnitude, table, positions, seq_rows, block_table, table_stride, (elem_t*)cache, page_size, (elem_t*)q_out, write_kv);
+      magnitude, table, positions, seq_rows, block_table, table_stride, (elem_t*)cache, page_size, (elem_t*)q_out, write_kv, q_temp_coef,
+      q_temp_every);
   AXK_LAUNCH_CHECK("heads_prepare");
   return 0;
 }
@@ -754,7 +774,7 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
                                     void* out, int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
                                     int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale,
                                     float eps, const int32_t* tiles, int n_tiles, float* partial, long partial_floats,
-                                    void* stream) {
+                                    float sink, int gate_per_head, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0,
               "masked_attention: bad sizes T=%d heads=%d kv heads=%d dim=%d vdim=%d page=%d", n_tokens, heads, kv_heads, dim, vdim,
               page_size);
@@ -776,7 +796,7 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
 #define MA_LAUNCH(MAPS, DT, KC)                                                                                                 \
   rc = launch_masked_mfma<MAPS, DT, KC>(q, cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, out, tiles, nt, \
                                    heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda,        \
-                                   out_scale, eps, partial, (hipStream_t)stream)
+                                   out_scale, eps, partial, sink * 1.4426950408889634f, gate_per_head, (hipStream_t)stream)
     int rc = 0;
     // register tiles by the sizes: chunks of 32 key dims (2, 4 or 8), tiles of 16 value dims (4, 8 or 16)
 #define MA_BY_DIM(MAPS, DT)                                                                  \
@@ -800,7 +820,8 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
   const size_t lds = (size_t)maps * dim * MA_WAVES * sizeof(float);
   masked_attention_kernel<<<(unsigned)((items + MA_WAVES - 1) / MA_WAVES), MA_WAVES * 64, lds, (hipStream_t)stream>>>(
       (const elem_t*)q, (const elem_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, (elem_t*)out,
-      n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps);
+      n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps, sink,
+      gate_per_head);
   AXK_LAUNCH_CHECK("masked_attention");
   return 0;
 }

@@ -75,14 +75,15 @@ __global__ void route_topk_wave_kernel(const float* __restrict__ logits, int n_t
 // score is the sum of its two largest choice scores (of its one, if it has one expert), only experts
 // of the `keep` best groups can be chosen (of equal groups the lower), and among those the `top`
 // largest choice scores win (of equal ones the lower expert).  weights_k = s_k / (sum of the chosen s,
-// added in the order chosen, + 1e-20) * scale.  A wave per token: lane l holds experts l, l + 64, ...
+// added in the order chosen, + 1e-20) * scale, or without `normalize` the score itself times scale.  Rows of
+// logits are logits_stride apart (further columns may hold other products of the same input).  A wave per token: lane l holds experts l, l + 64, ...
 // (up to 1,024) and, for the groups' scores, walks group l (up to 64 groups).
-__global__ void route_scored_wave_kernel(const float* __restrict__ logits, const float* __restrict__ correction, int n_tokens,
-                                         int n_experts, int top, int groups, int keep, float scale, int32_t* __restrict__ experts,
-                                         float* __restrict__ weights) {
+__global__ void route_scored_wave_kernel(const float* __restrict__ logits, long logits_stride, const float* __restrict__ correction,
+                                         int n_tokens, int n_experts, int top, int groups, int keep, float scale, int normalize,
+                                         int32_t* __restrict__ experts, float* __restrict__ weights) {
   const int t = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64, lane = threadIdx.x & 63;
   if (t >= n_tokens) return;
-  const float* z = logits + (long)t * n_experts;
+  const float* z = logits + (long)t * logits_stride;
   const int size = n_experts / groups;
   unsigned long long kept = ~0ull;
   if (groups > 1) {
@@ -129,7 +130,7 @@ __global__ void route_scored_wave_kernel(const float* __restrict__ logits, const
     sum += s;
     if (lane == k % 64) { mine = s; experts[(long)t * top + k] = at; }
   }
-  if (lane < top) weights[(long)t * top + lane] = (mine / (sum + 1e-20f)) * scale;
+  if (lane < top) weights[(long)t * top + lane] = normalize ? (mine / (sum + 1e-20f)) * scale : mine * scale;
 }
 
 // One block.  pairs p = t top + k in expert order -> sorted [n_pairs], with the token of each
@@ -171,16 +172,23 @@ route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_expert
 }
 
 // y[t, :] (+)= sum_k weights[t, k] rows[row of pair t top + k, :], k ascending; a pair's row is the pair
-// itself, or place_of[pair].
+// itself, or place_of[pair]; without weights the rows are added as they are.  extra (or null): a further
+// row a token, added last, times sigmoid(extra_gate[t extra_gate_stride]) if a gate is given.
 __global__ void route_combine_kernel(const float* __restrict__ rows, const float* __restrict__ weights, float* __restrict__ y,
-                                     int top, int width, int accumulate, const int32_t* __restrict__ place_of) {
+                                     int top, int width, int accumulate, const int32_t* __restrict__ place_of,
+                                     const float* __restrict__ extra, const float* __restrict__ extra_gate, long extra_gate_stride) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= width) return;
   float acc = accumulate ? y[(long)t * width + c] : 0.0f;
   for (int k = 0; k < top; ++k) {
     const long pair = (long)t * top + k;
-    acc = fmaf(weights[pair], rows[(place_of ? (long)place_of[pair] : pair) * width + c], acc);
+    const float row = rows[(place_of ? (long)place_of[pair] : pair) * width + c];
+    acc = weights ? fmaf(weights[pair], row, acc) : acc + row;
+  }
+  if (extra) {
+    const float e = extra[(long)t * width + c];
+    acc = extra_gate ? fmaf(1.0f / (1.0f + expf(-extra_gate[(long)t * extra_gate_stride])), e, acc) : acc + e;
   }
   y[(long)t * width + c] = acc;
 }
@@ -210,16 +218,18 @@ extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, 
   return 0;
 }
 
-extern "C" int axk_route_scored(const float* logits, const float* correction, int n_tokens, int n_experts, int top, int groups,
-                                int keep, float scale, int32_t* experts, float* weights, void* stream) {
+extern "C" int axk_route_scored(const float* logits, long logits_stride, const float* correction, int n_tokens, int n_experts,
+                                int top, int groups, int keep, float scale, int normalize, int32_t* experts, float* weights,
+                                void* stream) {
+  AXK_REQUIRE(logits_stride >= n_experts, "route_scored: rows of %ld logits for %d experts", logits_stride, n_experts);
   AXK_REQUIRE(n_tokens >= 0 && n_experts > 0 && n_experts <= 1024 && top > 0 && top <= 64,
               "route_scored: %d tokens, %d of %d experts (at most 64 of 1024)", n_tokens, top, n_experts);
   AXK_REQUIRE(groups >= 1 && groups <= 64 && n_experts % groups == 0 && keep >= 1 && keep <= groups &&
               (long)keep * (n_experts / groups) >= top,
               "route_scored: %d of %d groups of %d experts for %d a token", keep, groups, n_experts / (groups > 0 ? groups : 1), top);
   if (n_tokens == 0) return 0;
-  route_scored_wave_kernel<<<ceil_div(n_tokens, 4), 256, 0, (hipStream_t)stream>>>(logits, correction, n_tokens, n_experts, top, groups,
-                                                                                  keep, scale, experts, weights);
+  route_scored_wave_kernel<<<ceil_div(n_tokens, 4), 256, 0, (hipStream_t)stream>>>(logits, logits_stride, correction, n_tokens, n_experts, top,
+                                                                                  groups, keep, scale, normalize, experts, weights);
   AXK_LAUNCH_CHECK("route_scored");
   return 0;
 }
@@ -248,12 +258,14 @@ extern "C" int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts
 }
 
 extern "C" int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width,
-                                 int accumulate, const int32_t* place_of, void* stream) {
+                                 int accumulate, const int32_t* place_of, const float* extra, const float* extra_gate,
+                                 long extra_gate_stride, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && n_tokens <= 65535, "route_combine: T=%d top=%d width=%d", n_tokens, top,
               width);
   if (n_tokens == 0) return 0;
   dim3 grid(ceil_div(width, 256), n_tokens);
-  route_combine_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rows, weights, y, top, width, accumulate, place_of);
+  route_combine_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rows, weights, y, top, width, accumulate, place_of, extra,
+                                                              extra_gate, extra_gate_stride);
   AXK_LAUNCH_CHECK("route_combine");
   return 0;
 }

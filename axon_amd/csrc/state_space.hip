@@ -1,0 +1,264 @@
+// A selective state-space mixer in its recurrent form (the "state-space duality" layer of Mamba-2-like
+// models): per request and head a state S [N, P] of 32-bit floats, carried from token to token,
+//   dt_t = softplus(raw_t + dt_bias),  a_t = exp(-exp(A_log) dt_t),
+//   S_t = a_t S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t,
+// behind a short causal convolution with silu over the channels [x | B | C], and followed by a gate and
+// an RMS norm in equal parts.  Head h reads B and C of group h / (heads / groups).
+//
+// A request's state row holds two copies of (heads N P floats of S, head by head [N][P], then
+// [taps - 1][channels] of the convolution's last inputs, oldest first); zeros for a new request, which
+// is also what the convolution reads before the first token.  The state behind position p lives in copy
+// p & 1: a step whose first position is s reads copy (s - 1) & 1 and writes the copy of its last
+// position, so a step of one token never writes what it read and gives the same state and output if it
+// is run again (a decoding step is run once before it is captured into a graph).  The tokens of a
+// request are contiguous in a step and a request is in a step once, so two tokens belong to one request
+// iff their state slots (seq_rows) are equal.  Everything here is 32-bit in both builds but the
+// convolution's weights as stored and the normed output.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+__device__ inline float ss_silu(float z) { return z / (1.0f + expf(-z)); }
+__device__ inline float ss_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+// u[t, c] = act(bias[c] + sum_k w[c, k] in(t - (taps - 1 - k))) for the channels c of x (float32 rows
+// x_stride apart): the last column of w is the current token's; inputs before the step come from the state.
+// Threads behind the channels work out the heads' step sizes: terms[t, h] = (dt, a) from raw[t, h].
+__global__ void state_conv_kernel(const float* __restrict__ x, long x_stride, const elem_t* __restrict__ w,
+                                  const void* __restrict__ bias, int bias_is_f32, int silu, const float* __restrict__ state,
+                                  long state_stride, long copy_elems, long tail_at, const int32_t* __restrict__ positions,
+                                  const int32_t* __restrict__ seq_rows, float* __restrict__ u, int channels, int taps,
+                                  const float* __restrict__ raw, long raw_stride, const void* __restrict__ dt_bias,
+                                  int dt_bias_is_f32, const void* __restrict__ a_log, int a_log_is_f32,
+                                  float* __restrict__ terms, int heads) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) {
+    const int h = c - channels;
+    if (h < heads) {
+      const float dt = ss_softplus(raw[(long)t * raw_stride + h] + load_vec(dt_bias, dt_bias_is_f32, h));
+      terms[((long)t * heads + h) * 2] = dt;
+      terms[((long)t * heads + h) * 2 + 1] = expf(-(expf(load_vec(a_log, a_log_is_f32, h)) * dt));
+    }
+    return;
+  }
+  const int slot = seq_rows[t];
+  // how many earlier tokens of this step belong to the same request (up to taps - 1 matter)
+  int inside = 0;
+  while (inside < taps - 1 && t - inside - 1 >= 0 && seq_rows[t - inside - 1] == slot) ++inside;
+  // the copy behind the position before the request's first of this step
+  const int before = (positions[t] - inside + 1) & 1;
+  const float* kept = state + (long)slot * state_stride + (long)before * copy_elems + tail_at;      // [taps - 1][channels]
+  float acc = 0.0f;
+  for (int k = 0; k < taps; ++k) {
+    const int back = taps - 1 - k;            // the input `back` tokens before this one
+    float v;
+    if (back <= inside) v = x[(long)(t - back) * x_stride + c];
+    else v = kept[(long)(taps - 1 - (back - inside)) * channels + c];        // the (back - inside)-th last kept input
+    acc = fmaf(to_float(w[(long)c * taps + k]), v, acc);
+  }
+  if (bias) acc += load_vec(bias, bias_is_f32, c);
+  u[(long)t * channels + c] = silu ? ss_silu(acc) : acc;
+}
+
+// The walk.  grid (requests of the step, heads, blocks of 16 value dims); a block is 256 threads: sixteen
+// lanes side by side share a value dim p and hold the state's rows n = lane, lane + 16, ... of that
+// column (OWN each: N up to 16 OWN); four tokens' operands are asked for ahead of the chain that needs
+// them.  spans [n][3] = (slot, first token, tokens), or null: every token a request of its own (a
+// decoding step) in slot seq_rows[t].  u [T, channels] = [x: heads P | B: groups N | C: groups N] behind
+// the convolution; terms [T, heads, 2] = (dt, a).  y [T, heads P] float32.  The block (head 0, dims 0)
+// also brings the convolution's kept inputs up to date from conv_in (the convolution's inputs, float32
+// rows conv_in_stride apart).  A sum over n is sixteen partial chains in ascending n folded by a
+// butterfly: the same for a token however the request was cut into steps.
+#define SS_AHEAD 4
+template <int OWN>
+__global__ void __launch_bounds__(256)
+state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ terms, const void* __restrict__ d_skip,
+                        int d_is_f32, float* __restrict__ state, long state_stride, long copy_elems, long tail_at,
+                        const int32_t* __restrict__ spans, const int32_t* __restrict__ positions,
+                        const int32_t* __restrict__ seq_rows, const float* __restrict__ conv_in, long conv_in_stride,
+                        float* __restrict__ y, int heads, int groups, int P, int N, int channels, int taps) {
+  int slot, first, count;
+  if (spans) {
+    slot = spans[3 * blockIdx.x]; first = spans[3 * blockIdx.x + 1]; count = spans[3 * blockIdx.x + 2];
+  } else {
+    slot = seq_rows[blockIdx.x]; first = blockIdx.x; count = 1;
+  }
+  const int h = blockIdx.y, g = h / (heads / groups);
+  const int ns = threadIdx.x & 15, p = blockIdx.z * 16 + (threadIdx.x >> 4);
+  const bool has_p = p < P;
+  const int start = positions[first];
+  const float* from = state + (long)slot * state_stride + (long)((start + 1) & 1) * copy_elems;
+  float* to = state + (long)slot * state_stride + (long)((start + count - 1) & 1) * copy_elems;
+  const int inner = heads * P;
+  const long s_at = (long)h * N * P;
+  float S[OWN];
+#pragma unroll
+  for (int i = 0; i < OWN; ++i) {
+    const int n = ns + 16 * i;
+    S[i] = has_p && n < N ? from[s_at + (long)n * P + p] : 0.0f;
+  }
+  const float dskip = load_vec(d_skip, d_is_f32, h);
+  const long x_col = (long)h * P + (has_p ? p : 0), b_col = inner + (long)g * N, c_col = inner + (long)groups * N + (long)g * N;
+  int t = first;
+  for (; t + SS_AHEAD <= first + count; t += SS_AHEAD) {
+    float xs[SS_AHEAD], dt[SS_AHEAD], a[SS_AHEAD], B[SS_AHEAD][OWN], C[SS_AHEAD][OWN];
+#pragma unroll
+    for (int k = 0; k < SS_AHEAD; ++k) {
+      const float* row = u + (long)(t + k) * channels;
+      xs[k] = row[x_col];
+      dt[k] = terms[((long)(t + k) * heads + h) * 2];
+      a[k] = terms[((long)(t + k) * heads + h) * 2 + 1];
+#pragma unroll
+      for (int i = 0; i < OWN; ++i) {
+        const int n = min(ns + 16 * i, N - 1);          // rows beyond N hold zeros in S: what they meet does not count
+        B[k][i] = row[b_col + n];
+        C[k][i] = row[c_col + n];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < SS_AHEAD; ++k) {
+      const float dx = dt[k] * xs[k];
+      float part = 0.0f;
+#pragma unroll
+      for (int i = 0; i < OWN; ++i) {
+        S[i] = ns + 16 * i < N ? fmaf(a[k], S[i], dx * B[k][i]) : 0.0f;
+        part = fmaf(S[i], C[k][i], part);
+      }
+      part += __shfl_xor(part, 8, 64);
+      part += __shfl_xor(part, 4, 64);
+      part += __shfl_xor(part, 2, 64);
+      part += __shfl_xor(part, 1, 64);
+      if (ns == 0 && has_p) y[(long)(t + k) * inner + x_col] = fmaf(dskip, xs[k], part);
+    }
+  }
+  for (; t < first + count; ++t) {
+    const float* row = u + (long)t * channels;
+    const float x1 = row[x_col], dt1 = terms[((long)t * heads + h) * 2], a1 = terms[((long)t * heads + h) * 2 + 1];
+    const float dx = dt1 * x1;
+    float part = 0.0f;
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+      const int n = min(ns + 16 * i, N - 1);
+      S[i] = ns + 16 * i < N ? fmaf(a1, S[i], dx * row[b_col + n]) : 0.0f;
+      part = fmaf(S[i], row[c_col + n], part);
+    }
+    part += __shfl_xor(part, 8, 64);
+    part += __shfl_xor(part, 4, 64);
+    part += __shfl_xor(part, 2, 64);
+    part += __shfl_xor(part, 1, 64);
+    if (ns == 0 && has_p) y[(long)t * inner + x_col] = fmaf(dskip, x1, part);
+  }
+#pragma unroll
+  for (int i = 0; i < OWN; ++i) {
+    const int n = ns + 16 * i;
+    if (has_p && n < N) to[s_at + (long)n * P + p] = S[i];
+  }
+  if (blockIdx.y != 0 || blockIdx.z != 0) return;
+  // the convolution's last taps - 1 inputs: of (what was kept, this step's inputs) the last taps - 1; place
+  // i takes what lies `count` places later (where both copies are one: read before it is written, ascending)
+  float* kept = to + tail_at;
+  const float* kept_from = from + tail_at;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x)
+    for (int i = 0; i < taps - 1; ++i) {
+      const int at = i + count;
+      kept[(long)i * channels + c] = at < taps - 1 ? kept_from[(long)at * channels + c]
+                                                   : conv_in[(long)(first + at - (taps - 1)) * conv_in_stride + c];
+    }
+}
+
+// out[t, part] = ((v / sqrt(mean(v^2) + eps)) gain) with v = y[t, part] silu(z[t, part]): the gate first,
+// then the norm of each of `parts` equal parts of a row by its own root mean square.  A wave a (token, part).
+__global__ void __launch_bounds__(256)
+gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ z, long z_stride, const void* __restrict__ gain,
+                        int gain_is_f32, float eps, elem_t* __restrict__ out, int n_tokens, int width, int parts) {
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (item >= (long)n_tokens * parts) return;
+  const int t = (int)(item / parts), part = (int)(item % parts), size = width / parts;
+  const float* ys = y + (long)t * width + (long)part * size;
+  const float* zs = z + (long)t * z_stride + (long)part * size;
+  float ss = 0.0f;
+  for (int i = lane; i < size; i += 64) {
+    const float v = ys[i] * ss_silu(zs[i]);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)size + eps);
+  elem_t* dst = out + (long)t * width + (long)part * size;
+  for (int i = lane; i < size; i += 64) {
+    const float v = ys[i] * ss_silu(zs[i]);
+    dst[i] = from_float((v * inv) * load_vec(gain, gain_is_f32, part * size + i));
+  }
+}
+
+}  // namespace
+
+extern "C" int axk_state_conv(const float* x, long x_stride, const void* w, const void* bias, int bias_is_f32, int silu,
+                              const float* state, long state_stride, long copy_elems, long tail_at, const int32_t* positions,
+                              const int32_t* seq_rows, float* u, int n_tokens, int channels, int taps, const float* raw,
+                              long raw_stride, const void* dt_bias, int dt_bias_is_f32, const void* a_log, int a_log_is_f32,
+                              float* terms, int heads, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && channels > 0 && taps >= 1 && x_stride >= channels && heads >= 0,
+              "state_conv: bad sizes T=%d channels=%d taps=%d heads=%d row stride %ld", n_tokens, channels, taps, heads, x_stride);
+  AXK_REQUIRE(tail_at >= 0 && copy_elems >= tail_at + (long)(taps - 1) * channels && state_stride >= 2 * copy_elems,
+              "state_conv: a state row of %ld floats does not hold two copies of %ld with %d x %d kept inputs from %ld",
+              state_stride, copy_elems, taps - 1, channels, tail_at);
+  AXK_REQUIRE(heads == 0 || (raw != nullptr && dt_bias != nullptr && a_log != nullptr && terms != nullptr && raw_stride >= heads),
+              "state_conv: step sizes of %d heads need their inputs", heads);
+  AXK_REQUIRE(n_tokens <= 65535, "state_conv: %d tokens in one step (at most 65535)", n_tokens);
+  if (n_tokens == 0) return 0;
+  dim3 grid(ceil_div(channels + heads, 256), n_tokens);
+  state_conv_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(x, x_stride, (const elem_t*)w, bias, bias_is_f32, silu, state,
+                                                          state_stride, copy_elems, tail_at, positions, seq_rows, u, channels,
+                                                          taps, raw, raw_stride, dt_bias, dt_bias_is_f32, a_log, a_log_is_f32,
+                                                          terms, heads);
+  AXK_LAUNCH_CHECK("state_conv");
+  return 0;
+}
+
+extern "C" int axk_state_space_scan(const float* u, const float* terms, const void* d_skip, int d_is_f32, float* state,
+                                    long state_stride, long copy_elems, long tail_at, const int32_t* spans, int n_spans,
+                                    const int32_t* positions, const int32_t* seq_rows, const float* conv_in, long conv_in_stride,
+                                    float* y, int heads, int groups, int vdim, int n_state, int taps, void* stream) {
+  AXK_REQUIRE(n_spans >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && vdim > 0 && n_state > 0 && taps >= 1,
+              "state_space_scan: bad sizes spans=%d heads=%d groups=%d vdim=%d state=%d taps=%d", n_spans, heads, groups, vdim,
+              n_state, taps);
+  AXK_REQUIRE(n_state <= 256, "state_space_scan: a state of %d rows a head (at most 256)", n_state);
+  const int channels = heads * vdim + 2 * groups * n_state;
+  AXK_REQUIRE(tail_at >= (long)heads * n_state * vdim && copy_elems >= tail_at + (long)(taps - 1) * channels &&
+              state_stride >= 2 * copy_elems && conv_in_stride >= channels,
+              "state_space_scan: a state row of %ld floats does not hold two copies of %ld (%d x %d x %d, then %d x %d from %ld)",
+              state_stride, copy_elems, heads, n_state, vdim, taps - 1, channels, tail_at);
+  AXK_REQUIRE((spans != nullptr || seq_rows != nullptr) && positions != nullptr, "state_space_scan: neither spans nor slots, or no positions");
+  AXK_REQUIRE(n_spans <= 65535 * 32 && heads <= 65535 && ceil_div(vdim, 16) <= 65535, "state_space_scan: %d requests of %d heads", n_spans, heads);
+  if (n_spans == 0) return 0;
+  dim3 grid(n_spans, heads, ceil_div(vdim, 16));
+  hipStream_t s = (hipStream_t)stream;
+#define SS_LAUNCH(OWN)                                                                                                        \
+  state_space_scan_kernel<OWN><<<grid, 256, 0, s>>>(u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, \
+                                                    positions, seq_rows, conv_in, conv_in_stride, y, heads, groups, vdim,    \
+                                                    n_state, channels, taps)
+  if (n_state <= 16) SS_LAUNCH(1);
+  else if (n_state <= 32) SS_LAUNCH(2);
+  else if (n_state <= 64) SS_LAUNCH(4);
+  else if (n_state <= 128) SS_LAUNCH(8);
+  else SS_LAUNCH(16);
+#undef SS_LAUNCH
+  AXK_LAUNCH_CHECK("state_space_scan");
+  return 0;
+}
+
+extern "C" int axk_gated_group_norm(const float* y, const float* z, long z_stride, const void* gain, int gain_is_f32, float eps,
+                                    void* out, int n_tokens, int width, int parts, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && width > 0 && parts > 0 && width % parts == 0 && z_stride >= width,
+              "gated_group_norm: bad sizes T=%d width=%d parts=%d", n_tokens, width, parts);
+  if (n_tokens == 0) return 0;
+  const long items = (long)n_tokens * parts;
+  gated_group_norm_kernel<<<(unsigned)((items + 3) / 4), 256, 0, (hipStream_t)stream>>>(y, z, z_stride, gain, gain_is_f32, eps,
+                                                                                        (elem_t*)out, n_tokens, width, parts);
+  AXK_LAUNCH_CHECK("gated_group_norm");
+  return 0;
+}

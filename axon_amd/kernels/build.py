@@ -31,7 +31,7 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 
 KERNEL_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "attention_mfma.hip",
-                  "sampling.hip", "grouped_gemm.hip", "recurrent.hip", "latent_attention.hip", "masked_attention.hip", "moe.hip", "instances.hip",
+                  "sampling.hip", "grouped_gemm.hip", "recurrent.hip", "state_space.hip", "latent_attention.hip", "masked_attention.hip", "moe.hip", "instances.hip",
                   "support.hip"]
 # what a library built from a part's own kernel sources gets beside them (the error channel, the
 # list of its kernel instances)

@@ -80,18 +80,23 @@ _SIGNATURES = {
     "axk_clamped_glu": [c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_void_p],
     "axk_grouped_gemm_uses_mfma": [c_int, c_int, c_long, c_long],
     "axk_grouped_gemm": [c_void_p, c_int, c_long, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_long,
-                         c_void_p, c_void_p, c_long, c_int, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_void_p],
+                         c_void_p, c_void_p, c_long, c_int, c_void_p, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_int,
+                         c_int, c_int, c_int, c_int, c_void_p],
     "axk_route_topk": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "axk_route_scored": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p],
+    "axk_route_scored": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_void_p],
     "axk_route_max_tiles": [c_int, c_int, c_int],
     "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
-    "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
+    "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
     "axk_gather_rows": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                         c_int, c_void_p],
     "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
                        c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
+    "axk_state_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p,
+                       c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
+    "axk_state_space_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_long, c_long, c_long, c_void_p, c_int, c_void_p,
+                             c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_gated_group_norm": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int,
                            c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "axk_latent_query_rope": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -100,13 +105,15 @@ _SIGNATURES = {
     "axk_sum_norm": [c_void_p, c_float, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_layernorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
     "axk_softcap": [c_void_p, c_long, c_int, c_int, c_float, c_void_p],
+    "axk_scale_rows": [c_void_p, c_long, c_int, c_int, c_float, c_void_p],
+    "axk_add_scaled": [c_void_p, c_void_p, c_float, c_long, c_void_p],
     "axk_heads_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
                           c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
-                          c_int, c_void_p],
+                          c_int, c_float, c_int, c_void_p],
     "axk_masked_attention_uses_mfma": [c_int, c_int, c_int, c_int, c_int, c_int],
     "axk_masked_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_float,
-                             c_void_p, c_int, c_void_p, c_long, c_void_p],
+                             c_void_p, c_int, c_void_p, c_long, c_float, c_int, c_void_p],
     "axk_concat_round": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
@@ -222,7 +229,9 @@ class Kernels:
                   "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
                   "fill_i32", "fill_f32", "call", "norm_add", "round_rows", "activation", "clamped_glu", "grouped_gemm",
                   "route_topk", "route_sort", "route_combine", "gather_rows", "causal_conv", "gated_scan", "latent_prepare",
-                  "latent_query_rope", "latent_attention", "heads_prepare", "masked_attention", "concat_round")
+                  "latent_query_rope", "latent_attention", "heads_prepare", "masked_attention", "concat_round", "scale_rows",
+                  "add_scaled", "state_conv", "state_space_scan", "gated_group_norm", "route_scored", "sum_norm", "layernorm",
+                  "softcap")
     _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3, "grouped_gemm": 1}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
@@ -256,6 +265,12 @@ class Kernels:
     def _f32(t: torch.Tensor, what: str) -> None:
         if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
             raise KernelError(f"{what}: expected a contiguous float32 device tensor, got {t.dtype} on {t.device}")
+
+    @staticmethod
+    def _f32_rows(t: torch.Tensor, what: str) -> None:
+        """float32 rows that may lie apart (a view into the columns of a wider product's rows)."""
+        if t.dtype != torch.float32 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError(f"{what}: expected float32 rows on the device, got {t.dtype} {tuple(t.shape)} with strides {t.stride()}")
 
     @staticmethod
     def _i32(t: torch.Tensor, what: str) -> None:
@@ -711,6 +726,21 @@ class Kernels:
         self._check(self.lib.axk_softcap(_ptr(v), v.stride(0), v.shape[0], v.shape[1], float(cap), _stream()))
         return v
 
+    def scale_rows(self, v: torch.Tensor, factor: float) -> torch.Tensor:
+        """v *= factor in place on float32 rows."""
+        if v.dtype != torch.float32 or not v.is_cuda or v.dim() != 2 or v.stride(1) != 1:
+            raise KernelError(f"scale_rows: {tuple(v.shape)} {v.dtype} with strides {v.stride()}")
+        self._check(self.lib.axk_scale_rows(_ptr(v), v.stride(0), v.shape[0], v.shape[1], float(factor), _stream()))
+        return v
+
+    def add_scaled(self, x: torch.Tensor, y: torch.Tensor, factor: float = 1.0) -> torch.Tensor:
+        """x += factor * y on float32 tensors of one shape."""
+        self._f32(x, "add_scaled x"); self._f32(y, "add_scaled y")
+        if x.shape != y.shape or not x.is_contiguous() or not y.is_contiguous():
+            raise KernelError(f"add_scaled: {tuple(x.shape)} and {tuple(y.shape)}")
+        self._check(self.lib.axk_add_scaled(_ptr(x), _ptr(y), float(factor), x.numel(), _stream()))
+        return x
+
     def round_rows(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         self._f32(x, "round_rows x"); self._elem(out, "round_rows out")
         if out.numel() != x.numel() or not out.is_contiguous():
@@ -747,7 +777,7 @@ class Kernels:
     # ------------------------------------------------------------------ grouped products
     def grouped_gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, x_group_stride: int, out_group_stride: int,
                      bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, glu=None, routed=None,
-                     rows: Optional[int] = None, gate_per_group: bool = False) -> torch.Tensor:
+                     rows: Optional[int] = None, gate_per_group: bool = False, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         """out[orow(r), g ogs + n] = epilogue(sum_k x[xrow(r), g xgs + k] w[g, n, k] + bias[g, n]).
 
         x [rows, >= g xgs + K] float32 or compute dtype, rows may be strided; w [G, N, K] (with `glu`
@@ -757,7 +787,9 @@ class Kernels:
         max_tiles, x_rows, out_rows[, tile_rows]), int32 on the device: the listed rows (`rows` of them at
         most) meet the group their tile names; tile_rows (16, or 64: many rows a group) is what the list
         was made for.  `gate` (float32, out's shape): out is multiplied
-        by its sigmoid; with `gate_per_group` the gate holds one number a group, [rows, >= G]."""
+        by its sigmoid; with `gate_per_group` the gate holds one number a group, [rows, >= G].  `row_scale`
+        (float32, one number an out row): the sums are multiplied by it before bias and epilogue, as if the
+        row of x had been."""
         G, NW, K = w.shape
         N = NW // 2 if glu else NW
         self._elem(w, "grouped w")
@@ -787,12 +819,16 @@ class Kernels:
                     self._i32(t, "grouped_gemm routing")
             if x.shape[1] < K or out.shape[1] < N:
                 raise KernelError(f"grouped_gemm: x {tuple(x.shape)} / out {tuple(out.shape)} for {K} -> {N}")
+        if row_scale is not None:
+            self._f32(row_scale, "grouped_gemm row_scale")
+            if not row_scale.is_contiguous() or row_scale.numel() < (M if routed is not None else out.shape[0]):
+                raise KernelError(f"grouped_gemm: {row_scale.numel()} row factors for {M} rows")
         limit, alpha, shift = (tuple(glu) + (1.0,))[:3] if glu else (0.0, 0.0, 0.0)
         self._check(self.lib.axk_grouped_gemm(
             _ptr(x), 1 if x.dtype == torch.float32 else 0, x.stride(0), x_group_stride, _ptr(x_rows), _ptr(w), _ptr(bias),
             self._vec_flag(bias, "grouped bias"), _ptr(out), 1 if out.dtype == torch.float32 else 0, out.stride(0),
             out_group_stride, _ptr(out_rows), _ptr(gate), 0 if gate is None else gate.stride(0), 1 if gate_per_group else 0,
-            1 if glu else 0, float(limit), float(alpha), float(shift), _ptr(tiles), _ptr(n_tiles), int(max_tiles), int(tile_rows), M, N, K, G, _stream()))
+            _ptr(row_scale), 1 if glu else 0, float(limit), float(alpha), float(shift), _ptr(tiles), _ptr(n_tiles), int(max_tiles), int(tile_rows), M, N, K, G, _stream()))
         return out
 
     # ------------------------------------------------------------------ routing
@@ -804,19 +840,25 @@ class Kernels:
         self._check(self.lib.axk_route_topk(_ptr(logits), T, E, top, _ptr(experts), _ptr(weights), _stream()))
 
     def route_scored(self, logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float,
-                     experts: torch.Tensor, weights: torch.Tensor) -> None:
+                     experts: torch.Tensor, weights: torch.Tensor, normalize: bool = True, n_experts: Optional[int] = None) -> None:
         """Sigmoid scores, the choice by score + correction among the `keep` best of `groups` groups of
-        neighbouring experts, weights the chosen scores over their sum, times scale (axk_route_scored)."""
+        neighbouring experts, weights the chosen scores over their sum (without `normalize`: the scores
+        themselves), times scale (axk_route_scored).  `n_experts`: the leading columns of `logits` that
+        are router logits (all, unless given)."""
         self._f32(logits, "router logits"); self._i32(experts, "chosen experts"); self._f32(weights, "router weights")
         T, E = logits.shape
-        if experts.shape != (T, top) or weights.shape != (T, top) or not logits.is_contiguous():
+        if n_experts is not None:
+            if not 0 < n_experts <= E:
+                raise KernelError(f"route_scored: {n_experts} experts in rows of {E} logits")
+            E = int(n_experts)
+        if experts.shape != (T, top) or weights.shape != (T, top) or logits.stride(1) != 1:
             raise KernelError(f"route_scored: {tuple(experts.shape)} / {tuple(weights.shape)} for {T} x {top}")
         if correction is not None:
             self._f32(correction, "router correction")
             if correction.numel() != E:
                 raise KernelError(f"route_scored: a correction of {correction.numel()} for {E} experts")
-        self._check(self.lib.axk_route_scored(_ptr(logits), _ptr(correction), T, E, top, int(groups), int(keep), float(scale),
-                                              _ptr(experts), _ptr(weights), _stream()))
+        self._check(self.lib.axk_route_scored(_ptr(logits), logits.stride(0), _ptr(correction), T, E, top, int(groups), int(keep),
+                                              float(scale), 1 if normalize else 0, _ptr(experts), _ptr(weights), _stream()))
 
     def route_max_tiles(self, n_pairs: int, n_experts: int, tile_rows: int = 16) -> int:
         return int(self.lib.axk_route_max_tiles(n_pairs, n_experts, tile_rows))
@@ -842,16 +884,37 @@ class Kernels:
         self._check(self.lib.axk_gather_rows(_ptr(x), x.stride(0), _ptr(rows), _ptr(out), rows.numel(), x.shape[1], _stream()))
         return out
 
-    def route_combine(self, rows: torch.Tensor, weights: torch.Tensor, y: torch.Tensor, accumulate: bool = False,
-                      place_of: Optional[torch.Tensor] = None) -> torch.Tensor:
-        self._f32(rows, "expert rows"); self._f32(weights, "router weights"); self._f32(y, "combine y")
+    def route_combine(self, rows: torch.Tensor, weights: Optional[torch.Tensor], y: torch.Tensor, accumulate: bool = False,
+                      place_of: Optional[torch.Tensor] = None, top: Optional[int] = None, extra: Optional[torch.Tensor] = None,
+                      extra_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """y[t] (+)= sum_k weights[t, k] rows[t top + k] (weights None: all 1, `top` then says how many rows a
+        token) + extra[t] sigmoid(extra_gate[t]) (extra: float32 like y; extra_gate: a float32 column, one logit a
+        token, rows may be strided; None: no gate)."""
+        self._f32(rows, "expert rows"); self._f32(y, "combine y")
         if place_of is not None:
             self._i32(place_of, "combine place_of")
-        T, top = weights.shape
-        if rows.shape != (T * top, y.shape[1]) or y.shape[0] != T:
-            raise KernelError(f"route_combine: rows {tuple(rows.shape)}, weights {tuple(weights.shape)}, y {tuple(y.shape)}")
+        T = y.shape[0]
+        if weights is not None:
+            self._f32(weights, "router weights")
+            if weights.shape[0] != T or not weights.is_contiguous():
+                raise KernelError(f"route_combine: weights {tuple(weights.shape)} for {T} tokens")
+            top = weights.shape[1]
+        if top is None or rows.shape != (T * top, y.shape[1]) or not rows.is_contiguous() or not y.is_contiguous():
+            raise KernelError(f"route_combine: rows {tuple(rows.shape)}, {top} a token, y {tuple(y.shape)}")
+        gate_stride = 0
+        if extra is not None:
+            self._f32(extra, "combine extra")
+            if extra.shape != y.shape or not extra.is_contiguous():
+                raise KernelError(f"route_combine: extra {tuple(extra.shape)} beside y {tuple(y.shape)}")
+            if extra_gate is not None:
+                self._f32_rows(extra_gate, "combine extra gate")
+                if extra_gate.shape != (T, 1):
+                    raise KernelError(f"route_combine: a gate of {tuple(extra_gate.shape)} for {T} tokens")
+                gate_stride = extra_gate.stride(0)
+        elif extra_gate is not None:
+            raise KernelError("route_combine: a gate without the rows it gates")
         self._check(self.lib.axk_route_combine(_ptr(rows), _ptr(weights), _ptr(y), T, top, y.shape[1], 1 if accumulate else 0,
-                                               _ptr(place_of), _stream()))
+                                               _ptr(place_of), _ptr(extra), _ptr(extra_gate), gate_stride, _stream()))
         return y
 
     # ------------------------------------------------------------------ convolution and recurrence with per-request state
@@ -895,6 +958,72 @@ class Kernels:
                                             self._vec_flag(lam, "scan lam"), float(decay), _ptr(state), state.stride(0),
                                             _ptr(spans), n, _ptr(positions), _ptr(seq_rows), _ptr(out), C, int(block_width),
                                             int(taps), _ptr(terms), T, _stream()))
+        return out
+
+    # ------------------------------------------------------------------ a state-space mixer with per-request state
+    def state_conv(self, x, w, bias, state, copy_elems: int, tail_at: int, positions, seq_rows, u, silu: bool = True,
+                   raw=None, dt_bias=None, a_log=None, terms=None) -> torch.Tensor:
+        """u[t, c] = act(bias[c] + sum_k w[c, k] x(t - (taps - 1 - k))) over float32 rows x [T, C] (a view whose
+        rows may be strided), inputs before the step from the float32 state rows (two copies of `copy_elems`
+        floats, the kept inputs from `tail_at`: see csrc/state_space.hip).  With `raw` [T, heads] (float32, a
+        view), `dt_bias`, `a_log` and `terms` [T, heads, 2]: the heads' (dt, a) as well."""
+        self._f32_rows(x, "conv x"); self._elem(w, "conv w"); self._f32(state, "conv state"); self._f32(u, "conv u")
+        self._i32(seq_rows, "seq_rows"); self._i32(positions, "positions")
+        T, C = u.shape
+        if x.shape != (T, C) or w.dim() != 2 or w.shape[0] != C or not w.is_contiguous() or seq_rows.numel() != T:
+            raise KernelError(f"state_conv: x {tuple(x.shape)}, w {tuple(w.shape)}, u {tuple(u.shape)}")
+        if bias is not None and bias.numel() != C:
+            raise KernelError(f"state_conv: a bias of {bias.numel()} for {C} channels")
+        heads = 0
+        if raw is not None:
+            self._f32_rows(raw, "conv raw"); self._f32(terms, "conv terms")
+            heads = raw.shape[1]
+            if raw.shape[0] != T or raw.stride(1) != 1 or terms.shape != (T, heads, 2) or not terms.is_contiguous() \
+                    or dt_bias.numel() != heads or a_log.numel() != heads:
+                raise KernelError(f"state_conv: raw {tuple(raw.shape)}, terms {tuple(terms.shape)} for {heads} heads")
+        self._check(self.lib.axk_state_conv(
+            _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "conv bias"), 1 if silu else 0, _ptr(state),
+            state.stride(0), int(copy_elems), int(tail_at), _ptr(positions), _ptr(seq_rows), _ptr(u), T, C, w.shape[1],
+            _ptr(raw), 0 if raw is None else raw.stride(0), _ptr(dt_bias), self._vec_flag(dt_bias, "dt bias"), _ptr(a_log),
+            self._vec_flag(a_log, "A_log"), _ptr(terms), heads, _stream()))
+        return u
+
+    def state_space_scan(self, u, terms, d_skip, state, copy_elems: int, tail_at: int, spans, positions, seq_rows, conv_in, y,
+                         heads: int, groups: int, vdim: int, n_state: int, taps: int) -> torch.Tensor:
+        """The state-space recurrence over each request's tokens (see csrc/state_space.hip): u [T, heads vdim +
+        2 groups n_state] and terms [T, heads, 2] float32; spans int32 [n, 3] = (slot, first token, tokens) or None
+        (each token a request of its own in slot seq_rows[t]); conv_in: the convolution's inputs (float32, rows may
+        be strided), kept for the next step; y [T, heads vdim] float32."""
+        for t, what in ((u, "scan u"), (terms, "scan terms"), (state, "scan state"), (y, "scan y")):
+            self._f32(t, what)
+        self._f32_rows(conv_in, "scan conv_in")
+        self._i32(seq_rows, "seq_rows"); self._i32(positions, "positions")
+        T, C = u.shape
+        if C != heads * vdim + 2 * groups * n_state or not u.is_contiguous() or terms.shape != (T, heads, 2) \
+                or not terms.is_contiguous() or y.shape != (T, heads * vdim) or not y.is_contiguous() \
+                or conv_in.shape != (T, C) or conv_in.stride(1) != 1 or d_skip.numel() != heads or seq_rows.numel() != T:
+            raise KernelError(f"state_space_scan: u {tuple(u.shape)}, terms {tuple(terms.shape)}, y {tuple(y.shape)}")
+        if spans is not None:
+            self._i32(spans, "scan spans")
+            n = spans.shape[0]
+        else:
+            n = T
+        self._check(self.lib.axk_state_space_scan(
+            _ptr(u), _ptr(terms), _ptr(d_skip), self._vec_flag(d_skip, "D"), _ptr(state), state.stride(0), int(copy_elems),
+            int(tail_at), _ptr(spans), n, _ptr(positions), _ptr(seq_rows), _ptr(conv_in), conv_in.stride(0), _ptr(y), heads,
+            groups, vdim, n_state, taps, _stream()))
+        return y
+
+    def gated_group_norm(self, y, z, gain, eps: float, out, parts: int) -> torch.Tensor:
+        """out = rms in `parts` equal parts of (y silu(z)), times gain: y float32 [T, W], z float32 [T, W] (rows
+        may be strided), out [T, W] in the compute dtype."""
+        self._f32(y, "group norm y"); self._f32_rows(z, "group norm z"); self._elem(out, "group norm out")
+        T, W = y.shape
+        if z.shape != (T, W) or z.stride(1) != 1 or out.shape != (T, W) or not y.is_contiguous() or not out.is_contiguous() \
+                or gain.numel() != W or parts < 1 or W % parts:
+            raise KernelError(f"gated_group_norm: y {tuple(y.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)}, {parts} parts")
+        self._check(self.lib.axk_gated_group_norm(_ptr(y), _ptr(z), z.stride(0), _ptr(gain), self._vec_flag(gain, "group norm gain"),
+                                                  float(eps), _ptr(out), T, W, int(parts), _stream()))
         return out
 
     # ------------------------------------------------------------------ attention over a latent cache
@@ -962,9 +1091,9 @@ class Kernels:
             raise KernelError(f"{what}: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {row}]")
 
     def heads_prepare(self, proj, q_at, n_q, k_at, n_k, v_at, v_width, dim, q_gain, k_gain, eps, rot, neighbours, magnitude,
-                      table, positions, seq_rows, block_table, cache, page_size, q_out, write_kv=True) -> None:
+                      table, positions, seq_rows, block_table, cache, page_size, q_out, write_kv=True, q_temp=None) -> None:
         """The projections' float32 rows into queries (q_out) and the page's keys and values: see
-        axk_heads_prepare in csrc/api.h."""
+        axk_heads_prepare in csrc/api.h.  `q_temp` = (coef, every): a query's temperature by its position."""
         self._f32(proj, "heads proj"); self._f32(table, "rope table"); self._i32(positions, "positions")
         self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table"); self._elem(q_out, "heads q_out")
         T = positions.numel()
@@ -980,15 +1109,17 @@ class Kernels:
             _ptr(proj), proj.stride(0), q_at, n_q, k_at, n_k, v_at, v_width, dim, _ptr(q_gain), self._vec_flag(q_gain, "q gain"),
             _ptr(k_gain), self._vec_flag(k_gain, "k gain"), float(eps), rot, 1 if neighbours else 0, float(magnitude), _ptr(table),
             _ptr(positions), _ptr(seq_rows), _ptr(block_table), block_table.shape[-1], _ptr(cache), page_size, _ptr(q_out), T,
-            1 if write_kv else 0, _stream()))
+            1 if write_kv else 0, float(q_temp[0]) if q_temp else 0.0, int(q_temp[1]) if q_temp else 0, _stream()))
 
     def masked_attention_uses_mfma(self, heads, kv_heads, maps, dim, vdim, page_size) -> bool:
         return bool(self.lib.axk_masked_attention_uses_mfma(heads, kv_heads, maps, dim, vdim, page_size))
 
     def masked_attention(self, q, cache, block_table, positions, seq_rows, out, heads, kv_heads, maps, dim, vdim, page_size,
-                         mask, mask_size, scale, softcap=0.0, lam=0.0, out_scale=1.0, eps=0.0, gate=None, tiles=None) -> torch.Tensor:
+                         mask, mask_size, scale, softcap=0.0, lam=0.0, out_scale=1.0, eps=0.0, gate=None, tiles=None,
+                         sink=None, gate_per_head=False) -> torch.Tensor:
         """q [T, heads maps dim] -> out [T, heads vdim] (compute dtype): see axk_masked_attention in csrc/api.h.
-        `gate`: float32 rows (a view whose rows may be strided) of heads vdim gate logits, or None."""
+        `gate`: float32 rows (a view whose rows may be strided) of heads vdim gate logits (of heads logits with
+        `gate_per_head`), or None.  `sink`: the score of a key without a value in every softmax, or None."""
         self._elem(q, "attention q"); self._elem(out, "attention out")
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
         T = positions.numel()
@@ -1000,8 +1131,9 @@ class Kernels:
             raise KernelError(f"masked_attention: mask '{mask}' is not known ({', '.join(self.MASKS)})")
         gate_stride = 0
         if gate is not None:
-            if gate.dtype != torch.float32 or gate.shape != (T, heads * vdim) or gate.stride(1) != 1:
-                raise KernelError(f"masked_attention: gate {tuple(gate.shape)} {gate.dtype} is not float32 [{T}, {heads * vdim}]")
+            gw = heads if gate_per_head else heads * vdim
+            if gate.dtype != torch.float32 or gate.shape != (T, gw) or gate.stride(1) != 1:
+                raise KernelError(f"masked_attention: gate {tuple(gate.shape)} {gate.dtype} is not float32 [{T}, {gw}]")
             gate_stride = gate.stride(0)
         n_tiles = 0
         if tiles is not None:
@@ -1013,7 +1145,8 @@ class Kernels:
         self._check(self.lib.axk_masked_attention(
             _ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[-1], _ptr(positions), _ptr(seq_rows), _ptr(gate),
             gate_stride, _ptr(out), T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask], int(mask_size), float(scale),
-            float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _ptr(partial), need, _stream()))
+            float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _ptr(partial), need,
+            float("-inf") if sink is None else float(sink), 1 if gate_per_head else 0, _stream()))
         return out
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:

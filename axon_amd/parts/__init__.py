@@ -1,7 +1,8 @@
 from .base import (Block, CacheBinding, CacheSpec, FeedForward, Mixer, Norm, Part, PositionEncoding, StateSpec,
                    TensorDecl, build_block, build_part, register_block, register_embedding, register_feed_forward,
                    register_head, register_mixer, register_norm, register_position, register_stream, StreamEntry)
-from . import attention, block, embedding, latent_attention, masked_attention, mlp, moe, norm, recurrent, rope, stream  # noqa: F401  (registers the built-in parts)
+from . import (attention, block, embedding, latent_attention, masked_attention, mlp, moe, norm, paired, recurrent, rope,
+               state_space, stream)  # noqa: F401  (registers the built-in parts)
 
 __all__ = ["Block", "CacheBinding", "CacheSpec", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding",
            "StateSpec", "TensorDecl", "build_block", "build_part", "register_block", "register_embedding",

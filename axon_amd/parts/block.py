@@ -203,7 +203,39 @@ class PostNormBlock(Block):
         ctx.shared[ROUNDED_STREAM] = None if exact else (x, h)
 
 
+class ParallelBlock(Block):
+    """h = norm1(x); x += mixer(h) + feed_forward(h): one norm, and both sublayers read its output (a
+    layer may have no feed-forward).  Each sublayer adds into the 32-bit stream in the epilogue of its
+    last product."""
+    graph_safe = True
+    norm1_name = "norm1"
+
+    def __init__(self, norm_factory, mixer, feed_forward, prefix):
+        super().__init__(norm_factory, mixer, feed_forward, prefix)
+        self.norm1 = norm_factory(self.norm1_name)
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.feed_forward) if p is not None]
+
+    def tensors(self) -> List[TensorDecl]:
+        return [d for p in self.parts() for d in p.tensors()]
+
+    def load(self, store, rt) -> None:
+        for part in self.parts():
+            part.load(store, rt)
+
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
+        h = normed if normed is not None else self.norm1.forward(ctx, x)
+        self.mixer.forward(ctx, binding, h, x)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(ctx, h, x)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("parallel", ParallelBlock)
 register_block("prenorm_short_names", ShortNamedPreNormBlock)
 register_block("sublayer_norm", SublayerNormBlock)
 register_block("postnorm", PostNormBlock)

@@ -53,6 +53,7 @@ class LMHead(Part):
         self.tied_to = params.get("tied_to")
         self.tied = bool(params.get("tied", False))
         self.softcap = float(params.get("softcap", 0.0))      # > 0: logits = cap tanh(logits / cap)
+        self.scale = float(params.get("scale", 1.0))          # the logits are multiplied by it (32-bit), before the bend
         self.weight = None
         self.source_name = None      # the tensor the head was loaded from
 
@@ -81,6 +82,8 @@ class LMHead(Part):
         if out is None:
             out = torch.empty((h.shape[0], self.vocab), dtype=torch.float32, device=h.device)
         ctx.rt.k.gemm(h, self.weight, out, None, MODE_STORE_F32)
+        if self.scale != 1.0:
+            ctx.rt.k.scale_rows(out, self.scale)
         if self.softcap > 0.0:
             ctx.rt.k.softcap(out, self.softcap)
         return out

@@ -17,7 +17,12 @@ i // (heads / kv_heads).  What a configuration may turn on, each on its own:
   {"kind": "chunk", "size": n} (j <= i in the same chunk, floor(i / n) = floor(j / n), counted
   from position 0 of the request);
 * `softcap` c > 0: score <- c tanh(score / c), after the scale;
-* `gate`: the concatenated heads are multiplied by sigmoid(Wg h) before the output projection.
+* `sink` (a number): every softmax has one more key of that score, which has no value:
+  p_j = exp(s_j) / (exp(sink) + sum exp(s_j')); 0 adds one to the denominator;
+* `q_temp` = {"coef": c, "every": n}: the query at position p is multiplied by
+  1 + c ln(floor((p + 1) / n) + 1), in 32-bit, behind norm and rotation;
+* `gate`: the concatenated heads are multiplied by sigmoid(Wg h) before the output projection, a number
+  an element (true, or "elements": Wg has heads vdim rows) or a number a head ("heads": Wg has heads rows).
 
 All projections of h are one product into 32-bit rows; one kernel norms, rotates and stores
 (queries for the attention kernel, keys and values into the request's page, whose row holds a
@@ -27,7 +32,9 @@ into the residual stream.  With a window or chunks only the last `size` position
 so the cache manager may take back earlier pages.
 
 Parameters: `hidden_size`, `heads`, `kv_heads`, `dim`, `vdim`, `maps`, `diff`, `values`, `bias`,
-`qk_norm`, `eps`, `scale`, `softcap`, `mask`, `gate`, `position` (a PartSpec), `names`.
+`qk_norm`, `eps`, `scale`, `softcap`, `sink`, `q_temp`, `mask`, `gate`, `position` (a PartSpec), `names`.
+`forward(..., accumulate=False)` stores the 32-bit output instead of adding it (for a part that combines
+several mixers' outputs itself).
 """
 from __future__ import annotations
 
@@ -76,6 +83,7 @@ def attention_tiles(ctx, mask: str, size: int) -> Optional[torch.Tensor]:
 
 class MaskedAttention(Mixer):
     graph_safe = True
+    stores_output = True
 
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
@@ -84,6 +92,14 @@ class MaskedAttention(Mixer):
         self.dim, self.vdim, self.maps = int(p["dim"]), int(p["vdim"]), int(p.get("maps", 1))
         self.values = p.get("values", "projected")
         self.bias, self.qk_norm, self.gate = bool(p.get("bias", False)), bool(p.get("qk_norm", False)), bool(p.get("gate", False))
+        if p.get("gate") not in (None, False, True, "elements", "heads"):
+            raise ConfigError(f"gate {p.get('gate')!r} is not known (elements, heads)")
+        self.gate_per_head = p.get("gate") == "heads"
+        self.sink = None if p.get("sink") is None else float(p["sink"])
+        temp = p.get("q_temp")
+        self.q_temp = None if not temp else (float(temp["coef"]), int(temp["every"]))
+        if self.q_temp is not None and self.q_temp[1] < 1:
+            raise ConfigError(f"a query temperature every {self.q_temp[1]} positions")
         self.eps, self.scale = float(p.get("eps", 0.0)), float(p["scale"])
         self.softcap, self.diff = float(p.get("softcap") or 0.0), float(p.get("diff", 0.0))
         mask = p.get("mask") or {"kind": "causal"}
@@ -114,7 +130,8 @@ class MaskedAttention(Mixer):
         self.k_at = self.q_width
         self.v_at = self.k_at if self.values == "keys" else self.k_at + self.k_width
         self.g_at = self.k_at + self.k_width + (0 if self.values == "keys" else self.v_width)
-        self.proj_width = self.g_at + (self.o_width if self.gate else 0)
+        self.g_width = 0 if not self.gate else self.heads if self.gate_per_head else self.o_width
+        self.proj_width = self.g_at + self.g_width
         self.lam = 0.0
         self.q_gain = self.k_gain = self.b_proj = None
 
@@ -124,7 +141,7 @@ class MaskedAttention(Mixer):
 
     def tensors(self) -> List[TensorDecl]:
         n = self.n
-        rows = {"q": self.q_width, "k": self.k_width, "v": self.v_width, "g": self.o_width}
+        rows = {"q": self.q_width, "k": self.k_width, "v": self.v_width, "g": self.g_width}
         t = [TensorDecl(n[k], (rows[k], self.hidden)) for k in self._projections()]
         if self.bias:
             t += [TensorDecl(n[k] + ".b", (rows[k],), "bias") for k in self._projections() if k != "g"]
@@ -144,7 +161,7 @@ class MaskedAttention(Mixer):
         names = self._projections()
         self.w_proj = rt.k.prepare_weight(store.fused_matrix([n[k] for k in names]))
         if self.bias:
-            parts = [store.vector(n[k] + ".b").float() if k != "g" else torch.zeros(self.o_width, device=rt.device) for k in names]
+            parts = [store.vector(n[k] + ".b").float() if k != "g" else torch.zeros(self.g_width, device=rt.device) for k in names]
             self.b_proj = torch.cat(parts).contiguous()
         if self.qk_norm:
             self.q_gain, self.k_gain = store.vector(n["q"] + ".norm"), store.vector(n["k"] + ".norm")
@@ -162,7 +179,7 @@ class MaskedAttention(Mixer):
         """In steps of many rows the output projection's last kernel also writes the norm behind it."""
         return isinstance(self.w_o, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.o_width)
 
-    def forward(self, ctx, binding: CacheBinding, h, residual, following=None) -> None:
+    def forward(self, ctx, binding: CacheBinding, h, residual, following=None, accumulate: bool = True) -> None:
         k, T = ctx.rt.k, h.shape[0]
         group = ctx.cache.group(binding.group)
         (cache,) = group.layer(binding.index)
@@ -175,14 +192,18 @@ class MaskedAttention(Mixer):
         q = ctx.ws.take((T, self.q_width), ctx.rt.dtype)
         k.heads_prepare(proj, 0, self.n_q, self.k_at, self.n_k, self.v_at, self.v_width, self.dim, self.q_gain, self.k_gain,
                         self.eps, self.rot, neighbours, magnitude, table, ctx.positions, ctx.seq_rows, group.block_table, cache,
-                        group.page_size, q, binding.writes)
+                        group.page_size, q, binding.writes, q_temp=self.q_temp)
         att = ctx.ws.take((T, self.o_width), ctx.rt.dtype)
         tiles = None
         if k.masked_attention_uses_mfma(self.heads, self.kv_heads, self.maps, self.dim, self.vdim, group.page_size):
             tiles = attention_tiles(ctx, self.mask, self.mask_size)
         k.masked_attention(q, cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.heads, self.kv_heads, self.maps,
                            self.dim, self.vdim, group.page_size, self.mask, self.mask_size, self.scale, self.softcap, self.lam,
-                           1.0 - self.diff, self.eps, gate=proj[:, self.g_at:] if self.gate else None, tiles=tiles)
+                           1.0 - self.diff, self.eps, gate=proj[:, self.g_at:] if self.gate else None, tiles=tiles,
+                           sink=self.sink, gate_per_head=self.gate_per_head)
+        if not accumulate:          # the output itself, for a part that sums and norms on its own
+            k.gemm(att, self.w_o, residual, None, MODE_STORE_F32)
+            return
         k.gemm(att, self.w_o, residual, None, MODE_ADD_F32,
                following_norm=None if following is None else following.as_argument())
 

@@ -5,6 +5,9 @@ output side by side (the stream's columns first).  A model whose layers run seve
 it at the start of every pass, so that each pass sees the tokens again.  The two row sets are rounded
 to the compute dtype side by side by one small kernel, the product stores 32-bit rows into x.
 Parameters: `hidden_size`, `tensor`.
+
+"embedding_add": x <- x + factor x0, no tensor: a pass of a loop sees the tokens again by plain addition
+(32-bit).  Parameters: `factor` (default 1).
 """
 from __future__ import annotations
 
@@ -36,4 +39,16 @@ class EmbeddingMix(StreamEntry):
         k.gemm(both, self.weight, x, None, MODE_STORE_F32)
 
 
+class EmbeddingAdd(StreamEntry):
+    graph_safe = True
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.factor = float(params.get("factor", 1.0))
+
+    def forward(self, ctx, x, x0) -> None:
+        ctx.rt.k.add_scaled(x, x0, self.factor)
+
+
 register_stream("embedding_mix", EmbeddingMix)
+register_stream("embedding_add", EmbeddingAdd)
