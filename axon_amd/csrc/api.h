@@ -366,17 +366,18 @@ int axk_heads_prepare(const float* proj, long stride, int q_at, int n_q, int k_a
 // one a head.  sink > -inf: the softmax's sum also holds exp(sink), a key of that score without a value.  tiles (int32 [n_tiles, 2]: first token,
 // count; up to 16 consecutive tokens of one request each) or null (every token a tile of its own) are
 // what the matrix-core kernel works on where axk_masked_attention_uses_mfma says 1.
-// partial: axk_masked_attention_workspace floats (steps of few tokens under a window or in chunks: the
-// blocks of 64 positions of a single token then run side by side and a second launch folds them), or null.
+// partial: axk_masked_attention_workspace floats (steps of few tokens: the blocks of 64 positions of a single token
+// then run side by side and a second launch folds them; with mask_kind 0 as many blocks as `span`, the positions
+// the step's longest row sees, make: 0 there means no such split), or null.
 int axk_masked_attention_uses_mfma(int heads, int kv_heads, int maps, int dim, int vdim, int page_size);
 long axk_masked_attention_workspace(int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
-                                    int mask_kind, int mask_size);
+                                    int mask_kind, int mask_size, int span);
 int axk_masked_attention(const void* q, const void* cache, const int32_t* block_table, int table_stride,
                          const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
                          int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size, int mask_kind,
                          int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
                          const int32_t* tiles, int n_tiles, float* partial, long partial_floats, float sink, int gate_per_head,
-                         void* stream);
+                         int span, void* stream);
 
 #ifdef __cplusplus
 }

@@ -677,9 +677,11 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
                       gate_per_head);
 }
 
-// Blocks of positions a single token can touch under its mask (0: no bound).
-static int masked_chunks(int mask_kind, int mask_size) {
-  return mask_kind == MASK_CAUSAL ? 0 : (mask_size + 62) / 64 + 1;
+// Blocks of positions a single token can touch under its mask (0: no bound known).  Without a window or chunks
+// the bound is the step's: `span`, the positions its longest row sees.
+static int masked_chunks(int mask_kind, int mask_size, int span) {
+  if (mask_kind == MASK_CAUSAL) return span > 0 ? (span + 63) / 64 : 0;
+  return (mask_size + 62) / 64 + 1;
 }
 
 template <int MAPS, int DT, int KC>
@@ -687,7 +689,7 @@ static int launch_masked_mfma(const void* q, const void* cache, const int32_t* b
                               const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
                               const int32_t* tiles, int n_tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
                               int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
-                              float* partial, float sink_log2, int gate_per_head, hipStream_t stream) {
+                              float* partial, int span, float sink_log2, int gate_per_head, hipStream_t stream) {
   const int grp = heads / kv_heads;
   const size_t lds = ((size_t)64 * (MAPS * dim + 8) + (size_t)vdim * (64 + 8)) * sizeof(bf16_t);
   if (tiles != nullptr && partial == nullptr && KC <= 4 && DT <= 8 && lds <= 64 * 1024) {
@@ -708,7 +710,7 @@ static int launch_masked_mfma(const void* q, const void* cache, const int32_t* b
             sink_log2, gate_per_head);
     return 0;
   }
-  const int n_chunks = partial ? masked_chunks(mask_kind, mask_size) : 1;
+  const int n_chunks = partial ? masked_chunks(mask_kind, mask_size, span) : 1;
   masked_attention_mfma_kernel<MAPS, DT, KC><<<dim3(n_tiles, heads, n_chunks), 64, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, (bf16_t*)out, tiles,
       heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps, partial, n_chunks,
@@ -754,14 +756,15 @@ extern "C" int axk_masked_attention_uses_mfma(int heads, int kv_heads, int maps,
 #endif
 }
 
-// Steps of few tokens under a window or in chunks: the blocks of 64 positions of a single token run side
-// by side and a second launch folds them; the floats of the workspace that takes (0: a wave walks its
+// Steps of few tokens: the blocks of 64 positions of a single token run side by side and a second launch folds
+// them (under a window or in chunks as many blocks as the mask lets a token touch; else as many as `span`
+// positions, what the step's longest row sees, make); the floats of the workspace that takes (0: a wave walks its
 // token's blocks itself).
 extern "C" long axk_masked_attention_workspace(int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
-                                               int mask_kind, int mask_size) {
+                                               int mask_kind, int mask_size, int span) {
 #if AXON_BF16
   if (!axk_masked_attention_uses_mfma(heads, kv_heads, maps, dim, vdim, page_size)) return 0;
-  const int chunks = masked_chunks(mask_kind, mask_size);
+  const int chunks = masked_chunks(mask_kind, mask_size, span);
   if (chunks < 3 || (long)n_tokens * kv_heads >= 512) return 0;
   return (long)n_tokens * heads * chunks * maps * (vdim + 2);
 #else
@@ -774,7 +777,7 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
                                     void* out, int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
                                     int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale,
                                     float eps, const int32_t* tiles, int n_tiles, float* partial, long partial_floats,
-                                    float sink, int gate_per_head, void* stream) {
+                                    float sink, int gate_per_head, int span, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0,
               "masked_attention: bad sizes T=%d heads=%d kv heads=%d dim=%d vdim=%d page=%d", n_tokens, heads, kv_heads, dim, vdim,
               page_size);
@@ -789,14 +792,14 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
       ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
     AXK_REQUIRE(tiles == nullptr || n_tiles > 0, "masked_attention: a list of %d tiles", n_tiles);
     const int nt = tiles ? n_tiles : n_tokens;
-    const long need = axk_masked_attention_workspace(n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size);
+    const long need = axk_masked_attention_workspace(n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size, span);
     AXK_REQUIRE(partial == nullptr || partial_floats >= need, "masked_attention: a workspace of %ld floats, %ld needed",
                 partial_floats, need);
     if (need == 0) partial = nullptr;
 #define MA_LAUNCH(MAPS, DT, KC)                                                                                                 \
   rc = launch_masked_mfma<MAPS, DT, KC>(q, cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, out, tiles, nt, \
                                    heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda,        \
-                                   out_scale, eps, partial, sink * 1.4426950408889634f, gate_per_head, (hipStream_t)stream)
+                                   out_scale, eps, partial, span, sink * 1.4426950408889634f, gate_per_head, (hipStream_t)stream)
     int rc = 0;
     // register tiles by the sizes: chunks of 32 key dims (2, 4 or 8), tiles of 16 value dims (4, 8 or 16)
 #define MA_BY_DIM(MAPS, DT)                                                                  \

@@ -64,18 +64,36 @@ __global__ void state_conv_kernel(const float* __restrict__ x, long x_stride, co
   u[(long)t * channels + c] = silu ? ss_silu(acc) : acc;
 }
 
-// The walk.  grid (requests of the step, heads, blocks of 16 value dims); a block is 256 threads: sixteen
+// The sum over the sixteen lanes of a row, in every lane of the row, by lane permutations of the adder (pairs,
+// quads, halves of the row, the row): a fixed order.
+__device__ inline float ss_row_sum(float v) {
+#define SS_DPP(val, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, val), ctrl, 0xf, 0xf, false))
+  v += SS_DPP(v, 0xb1);     // quad_perm [1, 0, 3, 2]
+  v += SS_DPP(v, 0x4e);     // quad_perm [2, 3, 0, 1]
+  v += SS_DPP(v, 0x141);    // row_half_mirror
+  v += SS_DPP(v, 0x140);    // row_mirror
+#undef SS_DPP
+  return v;
+}
+
+// The walk.  grid (requests of the step, heads, blocks of 8 value dims); a block is 128 threads: sixteen
 // lanes side by side share a value dim p and hold the state's rows n = lane, lane + 16, ... of that
-// column (OWN each: N up to 16 OWN); four tokens' operands are asked for ahead of the chain that needs
-// them.  spans [n][3] = (slot, first token, tokens), or null: every token a request of its own (a
-// decoding step) in slot seq_rows[t].  u [T, channels] = [x: heads P | B: groups N | C: groups N] behind
-// the convolution; terms [T, heads, 2] = (dt, a).  y [T, heads P] float32.  The block (head 0, dims 0)
-// also brings the convolution's kept inputs up to date from conv_in (the convolution's inputs, float32
-// rows conv_in_stride apart).  A sum over n is sixteen partial chains in ascending n folded by a
-// butterfly: the same for a token however the request was cut into steps.
+// column (OWN each: N up to 16 OWN).  The operands of four tokens are asked for while the four before
+// them are worked on.  spans [n][3] = (slot, first token, tokens), or null: every token a request of its
+// own (a decoding step) in slot seq_rows[t].  u [T, channels] = [x: heads P | B: groups N | C: groups N]
+// behind the convolution; terms [T, heads, 2] = (dt, a).  y [T, heads P] float32.  The block (head 0,
+// dims 0) also brings the convolution's kept inputs up to date from conv_in (the convolution's inputs,
+// float32 rows conv_in_stride apart).  A sum over n is sixteen partial chains in ascending n folded in a
+// fixed order: the same for a token however the request was cut into steps.
 #define SS_AHEAD 4
+#define SS_THREADS 128
 template <int OWN>
-__global__ void __launch_bounds__(256)
+struct SsOperands {
+  float x[SS_AHEAD], dt[SS_AHEAD], a[SS_AHEAD], B[SS_AHEAD][OWN], C[SS_AHEAD][OWN];
+};
+
+template <int OWN>
+__global__ void __launch_bounds__(SS_THREADS)
 state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ terms, const void* __restrict__ d_skip,
                         int d_is_f32, float* __restrict__ state, long state_stride, long copy_elems, long tail_at,
                         const int32_t* __restrict__ spans, const int32_t* __restrict__ positions,
@@ -88,7 +106,7 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
     slot = seq_rows[blockIdx.x]; first = blockIdx.x; count = 1;
   }
   const int h = blockIdx.y, g = h / (heads / groups);
-  const int ns = threadIdx.x & 15, p = blockIdx.z * 16 + (threadIdx.x >> 4);
+  const int ns = threadIdx.x & 15, p = blockIdx.z * (SS_THREADS / 16) + (threadIdx.x >> 4);
   const bool has_p = p < P;
   const int start = positions[first];
   const float* from = state + (long)slot * state_stride + (long)((start + 1) & 1) * copy_elems;
@@ -96,61 +114,55 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
   const int inner = heads * P;
   const long s_at = (long)h * N * P;
   float S[OWN];
+  int n_of[OWN];
 #pragma unroll
   for (int i = 0; i < OWN; ++i) {
     const int n = ns + 16 * i;
     S[i] = has_p && n < N ? from[s_at + (long)n * P + p] : 0.0f;
+    n_of[i] = min(n, N - 1);            // rows beyond N hold zeros in S: what they meet does not count
   }
   const float dskip = load_vec(d_skip, d_is_f32, h);
   const long x_col = (long)h * P + (has_p ? p : 0), b_col = inner + (long)g * N, c_col = inner + (long)groups * N + (long)g * N;
-  int t = first;
-  for (; t + SS_AHEAD <= first + count; t += SS_AHEAD) {
-    float xs[SS_AHEAD], dt[SS_AHEAD], a[SS_AHEAD], B[SS_AHEAD][OWN], C[SS_AHEAD][OWN];
+  const int last = first + count;
+  auto fetch = [&](SsOperands<OWN>& o, int t0) {
 #pragma unroll
     for (int k = 0; k < SS_AHEAD; ++k) {
-      const float* row = u + (long)(t + k) * channels;
-      xs[k] = row[x_col];
-      dt[k] = terms[((long)(t + k) * heads + h) * 2];
-      a[k] = terms[((long)(t + k) * heads + h) * 2 + 1];
+      const int t = min(t0 + k, last - 1);             // behind the last token: the last again, not used
+      const float* row = u + (long)t * channels;
+      o.x[k] = row[x_col];
+      o.dt[k] = terms[((long)t * heads + h) * 2];
+      o.a[k] = terms[((long)t * heads + h) * 2 + 1];
 #pragma unroll
       for (int i = 0; i < OWN; ++i) {
-        const int n = min(ns + 16 * i, N - 1);          // rows beyond N hold zeros in S: what they meet does not count
-        B[k][i] = row[b_col + n];
-        C[k][i] = row[c_col + n];
+        o.B[k][i] = row[b_col + n_of[i]];
+        o.C[k][i] = row[c_col + n_of[i]];
       }
     }
+  };
+  auto work = [&](const SsOperands<OWN>& o, int t0) {
 #pragma unroll
     for (int k = 0; k < SS_AHEAD; ++k) {
-      const float dx = dt[k] * xs[k];
-      float part = 0.0f;
+      if (t0 + k < last) {
+        const float dx = o.dt[k] * o.x[k];
+        float part = 0.0f;
 #pragma unroll
-      for (int i = 0; i < OWN; ++i) {
-        S[i] = ns + 16 * i < N ? fmaf(a[k], S[i], dx * B[k][i]) : 0.0f;
-        part = fmaf(S[i], C[k][i], part);
+        for (int i = 0; i < OWN; ++i) {
+          S[i] = ns + 16 * i < N ? fmaf(o.a[k], S[i], dx * o.B[k][i]) : 0.0f;
+          part = fmaf(S[i], o.C[k][i], part);
+        }
+        part = ss_row_sum(part);
+        if (ns == 0 && has_p) y[(long)(t0 + k) * inner + x_col] = fmaf(dskip, o.x[k], part);
       }
-      part += __shfl_xor(part, 8, 64);
-      part += __shfl_xor(part, 4, 64);
-      part += __shfl_xor(part, 2, 64);
-      part += __shfl_xor(part, 1, 64);
-      if (ns == 0 && has_p) y[(long)(t + k) * inner + x_col] = fmaf(dskip, xs[k], part);
     }
-  }
-  for (; t < first + count; ++t) {
-    const float* row = u + (long)t * channels;
-    const float x1 = row[x_col], dt1 = terms[((long)t * heads + h) * 2], a1 = terms[((long)t * heads + h) * 2 + 1];
-    const float dx = dt1 * x1;
-    float part = 0.0f;
-#pragma unroll
-    for (int i = 0; i < OWN; ++i) {
-      const int n = min(ns + 16 * i, N - 1);
-      S[i] = ns + 16 * i < N ? fmaf(a1, S[i], dx * row[b_col + n]) : 0.0f;
-      part = fmaf(S[i], row[c_col + n], part);
-    }
-    part += __shfl_xor(part, 8, 64);
-    part += __shfl_xor(part, 4, 64);
-    part += __shfl_xor(part, 2, 64);
-    part += __shfl_xor(part, 1, 64);
-    if (ns == 0 && has_p) y[(long)t * inner + x_col] = fmaf(dskip, x1, part);
+  };
+  SsOperands<OWN> even, odd;
+  fetch(even, first);
+  for (int t = first; t < last; t += 2 * SS_AHEAD) {
+    if (t + SS_AHEAD < last) fetch(odd, t + SS_AHEAD);
+    work(even, t);
+    if (t + SS_AHEAD >= last) break;
+    if (t + 2 * SS_AHEAD < last) fetch(even, t + 2 * SS_AHEAD);
+    work(odd, t + SS_AHEAD);
   }
 #pragma unroll
   for (int i = 0; i < OWN; ++i) {
@@ -171,24 +183,35 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
 }
 
 // out[t, part] = ((v / sqrt(mean(v^2) + eps)) gain) with v = y[t, part] silu(z[t, part]): the gate first,
-// then the norm of each of `parts` equal parts of a row by its own root mean square.  A wave a (token, part).
+// then the norm of each of `parts` equal parts of a row by its own root mean square.  A block a (token, part):
+// a strided chain a thread, a butterfly a wave, the four waves in order.
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ z, long z_stride, const void* __restrict__ gain,
-                        int gain_is_f32, float eps, elem_t* __restrict__ out, int n_tokens, int width, int parts) {
-  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (item >= (long)n_tokens * parts) return;
-  const int t = (int)(item / parts), part = (int)(item % parts), size = width / parts;
+                        int gain_is_f32, float eps, elem_t* __restrict__ out, int width, int parts) {
+  __shared__ float partial[256 / AXON_WAVE];
+  const int t = blockIdx.x / parts, part = blockIdx.x % parts, size = width / parts;
   const float* ys = y + (long)t * width + (long)part * size;
   const float* zs = z + (long)t * z_stride + (long)part * size;
+  float kept[4];                      // parts of up to 1,024 values are read once
   float ss = 0.0f;
-  for (int i = lane; i < size; i += 64) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    kept[c] = i < size ? ys[i] * ss_silu(zs[i]) : 0.0f;
+    ss = fmaf(kept[c], kept[c], ss);
+  }
+  for (int i = threadIdx.x + 1024; i < size; i += 256) {
     const float v = ys[i] * ss_silu(zs[i]);
     ss = fmaf(v, v, ss);
   }
-  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)size + eps);
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, partial) / (float)size + eps);
   elem_t* dst = out + (long)t * width + (long)part * size;
-  for (int i = lane; i < size; i += 64) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    if (i < size) dst[i] = from_float((kept[c] * inv) * load_vec(gain, gain_is_f32, part * size + i));
+  }
+  for (int i = threadIdx.x + 1024; i < size; i += 256) {
     const float v = ys[i] * ss_silu(zs[i]);
     dst[i] = from_float((v * inv) * load_vec(gain, gain_is_f32, part * size + i));
   }
@@ -233,12 +256,12 @@ extern "C" int axk_state_space_scan(const float* u, const float* terms, const vo
               "state_space_scan: a state row of %ld floats does not hold two copies of %ld (%d x %d x %d, then %d x %d from %ld)",
               state_stride, copy_elems, heads, n_state, vdim, taps - 1, channels, tail_at);
   AXK_REQUIRE((spans != nullptr || seq_rows != nullptr) && positions != nullptr, "state_space_scan: neither spans nor slots, or no positions");
-  AXK_REQUIRE(n_spans <= 65535 * 32 && heads <= 65535 && ceil_div(vdim, 16) <= 65535, "state_space_scan: %d requests of %d heads", n_spans, heads);
+  AXK_REQUIRE(n_spans <= 65535 * 32 && heads <= 65535 && ceil_div(vdim, SS_THREADS / 16) <= 65535, "state_space_scan: %d requests of %d heads", n_spans, heads);
   if (n_spans == 0) return 0;
-  dim3 grid(n_spans, heads, ceil_div(vdim, 16));
+  dim3 grid(n_spans, heads, ceil_div(vdim, SS_THREADS / 16));
   hipStream_t s = (hipStream_t)stream;
 #define SS_LAUNCH(OWN)                                                                                                        \
-  state_space_scan_kernel<OWN><<<grid, 256, 0, s>>>(u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, \
+  state_space_scan_kernel<OWN><<<grid, SS_THREADS, 0, s>>>(u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, \
                                                     positions, seq_rows, conv_in, conv_in_stride, y, heads, groups, vdim,    \
                                                     n_state, channels, taps)
   if (n_state <= 16) SS_LAUNCH(1);
@@ -256,9 +279,9 @@ extern "C" int axk_gated_group_norm(const float* y, const float* z, long z_strid
   AXK_REQUIRE(n_tokens >= 0 && width > 0 && parts > 0 && width % parts == 0 && z_stride >= width,
               "gated_group_norm: bad sizes T=%d width=%d parts=%d", n_tokens, width, parts);
   if (n_tokens == 0) return 0;
-  const long items = (long)n_tokens * parts;
-  gated_group_norm_kernel<<<(unsigned)((items + 3) / 4), 256, 0, (hipStream_t)stream>>>(y, z, z_stride, gain, gain_is_f32, eps,
-                                                                                        (elem_t*)out, n_tokens, width, parts);
+  AXK_REQUIRE((long)n_tokens * parts <= 2147483647L, "gated_group_norm: %d tokens in %d parts", n_tokens, parts);
+  gated_group_norm_kernel<<<(unsigned)((long)n_tokens * parts), 256, 0, (hipStream_t)stream>>>(y, z, z_stride, gain, gain_is_f32, eps,
+                                                                                               (elem_t*)out, width, parts);
   AXK_LAUNCH_CHECK("gated_group_norm");
   return 0;
 }

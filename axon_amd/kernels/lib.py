@@ -113,7 +113,7 @@ _SIGNATURES = {
     "axk_masked_attention_uses_mfma": [c_int, c_int, c_int, c_int, c_int, c_int],
     "axk_masked_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_float,
-                             c_void_p, c_int, c_void_p, c_long, c_float, c_int, c_void_p],
+                             c_void_p, c_int, c_void_p, c_long, c_float, c_int, c_int, c_void_p],
     "axk_concat_round": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
@@ -166,7 +166,7 @@ class Kernels:
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
         self.lib.axk_latent_attention_workspace.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_int]
         self.lib.axk_latent_attention_workspace.restype = ctypes.c_long
-        self.lib.axk_masked_attention_workspace.argtypes = [c_int] * 9
+        self.lib.axk_masked_attention_workspace.argtypes = [c_int] * 10
         self.lib.axk_masked_attention_workspace.restype = ctypes.c_long
         self.lib.axk_packed_elems.argtypes = [c_int, c_int]
         self.lib.axk_packed_elems.restype = ctypes.c_long
@@ -1116,10 +1116,12 @@ class Kernels:
 
     def masked_attention(self, q, cache, block_table, positions, seq_rows, out, heads, kv_heads, maps, dim, vdim, page_size,
                          mask, mask_size, scale, softcap=0.0, lam=0.0, out_scale=1.0, eps=0.0, gate=None, tiles=None,
-                         sink=None, gate_per_head=False) -> torch.Tensor:
+                         sink=None, gate_per_head=False, span=0) -> torch.Tensor:
         """q [T, heads maps dim] -> out [T, heads vdim] (compute dtype): see axk_masked_attention in csrc/api.h.
         `gate`: float32 rows (a view whose rows may be strided) of heads vdim gate logits (of heads logits with
-        `gate_per_head`), or None.  `sink`: the score of a key without a value in every softmax, or None."""
+        `gate_per_head`), or None.  `sink`: the score of a key without a value in every softmax, or None.  `span`
+        (causal masks): the positions the step's longest row sees, so that a step of few tokens can run a token's
+        blocks of positions side by side; 0: a wave walks them."""
         self._elem(q, "attention q"); self._elem(out, "attention out")
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
         T = positions.numel()
@@ -1140,13 +1142,13 @@ class Kernels:
             self._i32(tiles, "attention tiles")
             n_tiles = tiles.shape[0]
         need = int(self.lib.axk_masked_attention_workspace(T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask],
-                                                           int(mask_size)))
+                                                           int(mask_size), int(span)))
         partial = torch.empty(need, dtype=torch.float32, device=out.device) if need else None
         self._check(self.lib.axk_masked_attention(
             _ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[-1], _ptr(positions), _ptr(seq_rows), _ptr(gate),
             gate_stride, _ptr(out), T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask], int(mask_size), float(scale),
             float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _ptr(partial), need,
-            float("-inf") if sink is None else float(sink), 1 if gate_per_head else 0, _stream()))
+            float("-inf") if sink is None else float(sink), 1 if gate_per_head else 0, int(span), _stream()))
         return out
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:

@@ -174,6 +174,15 @@ class MaskedAttention(Mixer):
         if self.position is not None:
             self.position.load(store, rt)
 
+    SPAN_STEP = 512      # the positions a decoding step's longest row sees, rounded up to this: part of the step's shape
+
+    def decode_shape(self, positions):
+        """Without a window or chunks the blocks of positions that run side by side in a step of few tokens
+        depend on how long the contexts are: a captured graph is replayed for steps whose longest row sees as many."""
+        if self.mask != "causal":
+            return None
+        return ("masked_attention_span", -(-(max(positions) + 1) // self.SPAN_STEP) * self.SPAN_STEP)
+
     # ------------------------------------------------------------------ the step
     def finishes_following_norm(self, ctx) -> bool:
         """In steps of many rows the output projection's last kernel also writes the norm behind it."""
@@ -197,10 +206,13 @@ class MaskedAttention(Mixer):
         tiles = None
         if k.masked_attention_uses_mfma(self.heads, self.kv_heads, self.maps, self.dim, self.vdim, group.page_size):
             tiles = attention_tiles(ctx, self.mask, self.mask_size)
+        span = 0
+        if self.mask == "causal":
+            span = ctx.decode_shapes.get("masked_attention_span", 0) if ctx.decode_only else max(s.start_pos + s.q_len for s in ctx.spans)
         k.masked_attention(q, cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.heads, self.kv_heads, self.maps,
                            self.dim, self.vdim, group.page_size, self.mask, self.mask_size, self.scale, self.softcap, self.lam,
                            1.0 - self.diff, self.eps, gate=proj[:, self.g_at:] if self.gate else None, tiles=tiles,
-                           sink=self.sink, gate_per_head=self.gate_per_head)
+                           sink=self.sink, gate_per_head=self.gate_per_head, span=span)
         if not accumulate:          # the output itself, for a part that sums and norms on its own
             k.gemm(att, self.w_o, residual, None, MODE_STORE_F32)
             return

@@ -151,6 +151,23 @@ def _pikesun_attention_sizes(width, heads, q_rank, experts, top, expert_ff, dens
             "residual_mult": 1.0, "vocab": 32000, "width": width}
 
 
+# --design zugutar: four layer runs: a pair of mixers (attention with normed, partly rotated queries and keys, a sink
+# and a gate a head beside a selective state-space scan of the model's width), an attention layer without rotation whose
+# queries carry a temperature by position, and a pair run twice over (the embedding added before its second pass); every
+# layer with experts fed their score times the input beside a gated shared expert.  Beside it the closest design the
+# engine has, Pikesun (a recurrence with per-request state, attention, as many experts of the same width), and the dense
+# decoder of equal width.
+def _zugutar_sizes(width, heads, kv_heads, ss_heads, groups, experts, top, expert_ff, shared_ff):
+    both = {"type": "parallel", "mixer": {
+        "left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "rot": {"base": 10000.0, "dims": 64}},
+        "right": {"heads": ss_heads, "vdim": 64, "state": 128, "groups": groups, "conv": 4, "norm_groups": groups}}}
+    att = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                          "q_temp": {"coef": 0.1, "every": 1024}}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff}}
+    return {"architecture": "Zugutar", "layers": [dict(both, mlp=moe), dict(att, mlp=moe), dict(both, mlp=moe)],
+            "loop": {"start": 2, "stop": 3, "times": 2}, "logit_scale": 0.25, "norm": {"eps": 1e-6}, "vocab": 32000, "width": width}
+
+
 # design -> size -> the models measured side by side, the design's own first
 DESIGN_SIZES = {
     "pikesun": {
@@ -164,6 +181,11 @@ DESIGN_SIZES = {
                  ("pikesun", _pikesun_attention_sizes(2048, 16, 768, 32, 4, 704, 5632)), ("qwen2", _qwen_sizes(2048, 16, 2, 5632))],
         "4096": [("napizen", _napizen_sizes(4096, 32, 64, 6, 1408, 11008, 8, 4)),
                  ("pikesun", _pikesun_attention_sizes(4096, 32, 1536, 64, 6, 1408, 11008)), ("qwen2", _qwen_sizes(4096, 32, 8, 11008))]},
+    "zugutar": {
+        "2048": [("zugutar", _zugutar_sizes(2048, 16, 2, 32, 2, 32, 4, 704, 1408)),
+                 ("pikesun", _pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024)), ("qwen2", _qwen_sizes(2048, 16, 2, 5632))],
+        "4096": [("zugutar", _zugutar_sizes(4096, 32, 8, 64, 8, 64, 6, 1408, 2816)),
+                 ("pikesun", _pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048)), ("qwen2", _qwen_sizes(4096, 32, 8, 11008))]},
 }
 
 
@@ -228,7 +250,7 @@ def design(args, torch) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default="", choices=["", "pikesun", "figalorn", "napizen"], help="instead of the headline benchmark: prefill and "
+    ap.add_argument("--design", default="", choices=["", "pikesun", "figalorn", "napizen", "zugutar"], help="instead of the headline benchmark: prefill and "
                     "decoding of this design at sizes that resemble real models' layers, beside the dense decoder of equal size")
     ap.add_argument("--design-size", default="", help="with --design: only this size (2048 or 4096)")
     ap.add_argument("--gpus", type=int, default=1)
