@@ -84,7 +84,9 @@ __device__ inline float ss_row_sum(float v) {
 // behind the convolution; terms [T, heads, 2] = (dt, a).  y [T, heads P] float32.  The block (head 0,
 // dims 0) also brings the convolution's kept inputs up to date from conv_in (the convolution's inputs,
 // float32 rows conv_in_stride apart).  A sum over n is sixteen partial chains in ascending n folded in a
-// fixed order: the same for a token however the request was cut into steps.
+// fixed order: the same for a token however the request was cut into steps.  FULL: N is 16 OWN, so no row
+// of a lane lies beyond the state (a lane's rows of B and C are then one address and constant offsets, and
+// nothing has to be kept at zero: a wave of this kernel is bound by the instructions it issues a token).
 #define SS_AHEAD 4
 #define SS_THREADS 128
 template <int OWN>
@@ -92,7 +94,7 @@ struct SsOperands {
   float x[SS_AHEAD], dt[SS_AHEAD], a[SS_AHEAD], B[SS_AHEAD][OWN], C[SS_AHEAD][OWN];
 };
 
-template <int OWN>
+template <int OWN, bool FULL>
 __global__ void __launch_bounds__(SS_THREADS)
 state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ terms, const void* __restrict__ d_skip,
                         int d_is_f32, float* __restrict__ state, long state_stride, long copy_elems, long tail_at,
@@ -124,18 +126,21 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
   const float dskip = load_vec(d_skip, d_is_f32, h);
   const long x_col = (long)h * P + (has_p ? p : 0), b_col = inner + (long)g * N, c_col = inner + (long)groups * N + (long)g * N;
   const int last = first + count;
+  const long lane_b = b_col + ns, lane_c = c_col + ns;
   auto fetch = [&](SsOperands<OWN>& o, int t0) {
 #pragma unroll
     for (int k = 0; k < SS_AHEAD; ++k) {
       const int t = min(t0 + k, last - 1);             // behind the last token: the last again, not used
       const float* row = u + (long)t * channels;
+      const float* bp = row + lane_b;
+      const float* cp = row + lane_c;
       o.x[k] = row[x_col];
       o.dt[k] = terms[((long)t * heads + h) * 2];
       o.a[k] = terms[((long)t * heads + h) * 2 + 1];
 #pragma unroll
       for (int i = 0; i < OWN; ++i) {
-        o.B[k][i] = row[b_col + n_of[i]];
-        o.C[k][i] = row[c_col + n_of[i]];
+        o.B[k][i] = FULL ? bp[16 * i] : row[b_col + n_of[i]];
+        o.C[k][i] = FULL ? cp[16 * i] : row[c_col + n_of[i]];
       }
     }
   };
@@ -147,7 +152,7 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
         float part = 0.0f;
 #pragma unroll
         for (int i = 0; i < OWN; ++i) {
-          S[i] = ns + 16 * i < N ? fmaf(o.a[k], S[i], dx * o.B[k][i]) : 0.0f;
+          S[i] = FULL || ns + 16 * i < N ? fmaf(o.a[k], S[i], dx * o.B[k][i]) : 0.0f;
           part = fmaf(S[i], o.C[k][i], part);
         }
         part = ss_row_sum(part);
@@ -260,16 +265,20 @@ extern "C" int axk_state_space_scan(const float* u, const float* terms, const vo
   if (n_spans == 0) return 0;
   dim3 grid(n_spans, heads, ceil_div(vdim, SS_THREADS / 16));
   hipStream_t s = (hipStream_t)stream;
-#define SS_LAUNCH(OWN)                                                                                                        \
-  state_space_scan_kernel<OWN><<<grid, SS_THREADS, 0, s>>>(u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, \
-                                                    positions, seq_rows, conv_in, conv_in_stride, y, heads, groups, vdim,    \
-                                                    n_state, channels, taps)
-  if (n_state <= 16) SS_LAUNCH(1);
-  else if (n_state <= 32) SS_LAUNCH(2);
-  else if (n_state <= 64) SS_LAUNCH(4);
-  else if (n_state <= 128) SS_LAUNCH(8);
-  else SS_LAUNCH(16);
+#define SS_ARGS u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, positions, seq_rows, conv_in, conv_in_stride, y, \
+                heads, groups, vdim, n_state, channels, taps
+#define SS_LAUNCH(OWN)                                                                              \
+  {                                                                                                 \
+    if (n_state == 16 * OWN) state_space_scan_kernel<OWN, true><<<grid, SS_THREADS, 0, s>>>(SS_ARGS); \
+    else state_space_scan_kernel<OWN, false><<<grid, SS_THREADS, 0, s>>>(SS_ARGS);                  \
+  }
+  if (n_state <= 16) SS_LAUNCH(1)
+  else if (n_state <= 32) SS_LAUNCH(2)
+  else if (n_state <= 64) SS_LAUNCH(4)
+  else if (n_state <= 128) SS_LAUNCH(8)
+  else SS_LAUNCH(16)
 #undef SS_LAUNCH
+#undef SS_ARGS
   AXK_LAUNCH_CHECK("state_space_scan");
   return 0;
 }
