@@ -323,7 +323,7 @@ CUTS = lambda T, page: [[T], [page - 1] + [1] * 8 + [T - page - 7], [2, 1, 1, 3]
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,vdim,state,groups,conv,norm_groups", [(3, 5, 7, 1, 3, 3), (4, 32, 64, 2, 4, 2), (2, 24, 130, 2, 2, 1),
-                                                                      (1, 40, 16, 1, 1, 1), (6, 16, 200, 3, 5, 6)])
+                                                                      (1, 40, 16, 1, 1, 1), (6, 16, 200, 3, 5, 6), (8, 64, 128, 2, 4, 2)])
 def test_the_state_space_side_alone_in_portions(heads, vdim, state, groups, conv, norm_groups, dtype):
     """The scan with its state and the convolution's kept inputs carried across cuts of every kind: whole, a
     token at a time from the first token on (a state that starts from nothing), portions that end inside the
@@ -394,7 +394,8 @@ def check_attention(cfg, W, scope, plain, page, dtype, T, cut_sets, side=None):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,dims,page", [(3, 1, 10, 6, 4, 8), (8, 2, 32, 32, 32, 64), (4, 4, 64, 48, 32, 64),
-                                                               (1, 1, 24, 40, 0, 16), (6, 3, 48, 16, 48, 128)])
+                                                               (1, 1, 24, 40, 0, 16), (6, 3, 48, 16, 48, 128), (8, 2, 128, 128, 64, 64),
+                                                               (32, 2, 64, 64, 64, 64), (4, 1, 256, 192, 128, 64)])
 def test_the_attention_side_with_a_sink_and_a_gate_a_head(heads, kv_heads, dim, vdim, dims, page, dtype):
     cfg = one_layer(64, pair(left(heads, kv_heads, dim, vdim, dims=dims, base=100.0), right(1, 8, 8)))
     W = {k: v for k, v in draw_weights(cfg, 31).items() if k.startswith("l0.mix.left.")}
@@ -420,7 +421,8 @@ def test_the_attention_side_with_a_sink_and_a_gate_a_head(heads, kv_heads, dim, 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,temp,page", [(4, 2, 6, 10, (0.7, 5), 8), (16, 16, 64, 16, (0.5, 64), 64),
-                                                               (2, 1, 24, 40, (0.25, 1), 16), (5, 5, 8, 8, None, 16), (8, 2, 32, 64, (1.0, 63), 64)])
+                                                               (2, 1, 24, 40, (0.25, 1), 16), (5, 5, 8, 8, None, 16), (8, 2, 32, 64, (1.0, 63), 64),
+                                                               (8, 2, 128, 128, (0.1, 128), 64), (40, 2, 64, 128, (0.5, 100), 64)])
 def test_attention_with_a_temperature_by_position_and_a_gate_an_element(heads, kv_heads, dim, vdim, temp, page, dtype):
     """Positions on both sides of every multiple of `every` (and of every - 1: the count goes by p + 1), in
     prompts and decoded."""
