@@ -304,7 +304,11 @@ int axk_gated_scan(const float* gates, const float* u, const void* y, long y_str
 // axk_state_space_scan: per request of the step (spans [n][3] = (slot, first token, tokens); null: each token a
 // request of its own in slot seq_rows[t]) and head, over its tokens in order, S = a S + dt B x^T, y = S^T C + D x
 // with u [T, channels] = [x: heads P | B: groups N | C: groups N]; y float32 [T, heads P]; then the state row is
-// brought up to date (S, and the convolution's inputs from conv_in, float32 rows conv_in_stride apart).
+// brought up to date (S, and the convolution's inputs from conv_in, float32 rows conv_in_stride apart).  With segs
+// ([n_segs][4] = (slot, first token, tokens, whether the request's first), the requests' stretches cut into
+// segments in order, none longer than longest_seg; spans5 [n][5] = (slot, first token, tokens, first segment, segments); ends float32 [n_segs,
+// heads, N, P]; cum float32 [T, heads]) the segments run side by side and two more launches fold their end states
+// and add what each segment's carried-in state gives its outputs (sums in another order than one walk's, by rounding).
 // axk_gated_group_norm: out[t] = rms in `parts` equal parts of (y[t] silu(z[t])), times gain; out elem [T, width].
 int axk_state_conv(const float* x, long x_stride, const void* w, const void* bias, int bias_is_f32, int silu, const float* state,
                    long state_stride, long copy_elems, long tail_at, const int32_t* positions, const int32_t* seq_rows, float* u,
@@ -313,7 +317,8 @@ int axk_state_conv(const float* x, long x_stride, const void* w, const void* bia
 int axk_state_space_scan(const float* u, const float* terms, const void* d_skip, int d_is_f32, float* state, long state_stride,
                          long copy_elems, long tail_at, const int32_t* spans, int n_spans, const int32_t* positions,
                          const int32_t* seq_rows, const float* conv_in, long conv_in_stride, float* y, int heads, int groups,
-                         int vdim, int n_state, int taps, void* stream);
+                         int vdim, int n_state, int taps, const int32_t* segs, int n_segs, int longest_seg, const int32_t* spans5,
+                         float* ends, float* cum, void* stream);
 int axk_gated_group_norm(const float* y, const float* z, long z_stride, const void* gain, int gain_is_f32, float eps, void* out,
                          int n_tokens, int width, int parts, void* stream);
 

@@ -100,9 +100,14 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
                         int d_is_f32, float* __restrict__ state, long state_stride, long copy_elems, long tail_at,
                         const int32_t* __restrict__ spans, const int32_t* __restrict__ positions,
                         const int32_t* __restrict__ seq_rows, const float* __restrict__ conv_in, long conv_in_stride,
-                        float* __restrict__ y, int heads, int groups, int P, int N, int channels, int taps) {
+                        float* __restrict__ y, int heads, int groups, int P, int N, int channels, int taps,
+                        const int32_t* __restrict__ segs, float* __restrict__ ends, float* __restrict__ cum) {
   int slot, first, count;
-  if (spans) {
+  bool from_state = true;
+  if (segs) {
+    slot = segs[4 * blockIdx.x]; first = segs[4 * blockIdx.x + 1]; count = segs[4 * blockIdx.x + 2];
+    from_state = segs[4 * blockIdx.x + 3] != 0;
+  } else if (spans) {
     slot = spans[3 * blockIdx.x]; first = spans[3 * blockIdx.x + 1]; count = spans[3 * blockIdx.x + 2];
   } else {
     slot = seq_rows[blockIdx.x]; first = blockIdx.x; count = 1;
@@ -120,7 +125,7 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
 #pragma unroll
   for (int i = 0; i < OWN; ++i) {
     const int n = ns + 16 * i;
-    S[i] = has_p && n < N ? from[s_at + (long)n * P + p] : 0.0f;
+    S[i] = from_state && has_p && n < N ? from[s_at + (long)n * P + p] : 0.0f;
     n_of[i] = min(n, N - 1);            // rows beyond N hold zeros in S: what they meet does not count
   }
   const float dskip = load_vec(d_skip, d_is_f32, h);
@@ -144,10 +149,14 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
       }
     }
   };
+  float decay = 1.0f;                  // of a segment: the product of its tokens' a so far
+  const bool tells_decay = cum != nullptr && blockIdx.z == 0 && threadIdx.x == 0;
   auto work = [&](const SsOperands<OWN>& o, int t0) {
 #pragma unroll
     for (int k = 0; k < SS_AHEAD; ++k) {
       if (t0 + k < last) {
+        decay *= o.a[k];
+        if (tells_decay) cum[(long)(t0 + k) * heads + h] = decay;
         const float dx = o.dt[k] * o.x[k];
         float part = 0.0f;
 #pragma unroll
@@ -169,6 +178,15 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
     if (t + 2 * SS_AHEAD < last) fetch(even, t + 2 * SS_AHEAD);
     work(odd, t + SS_AHEAD);
   }
+  if (segs) {                          // a segment's end state goes to the workspace; the fold brings the request's state up to date
+    float* end = ends + ((long)blockIdx.x * heads + h) * N * P;
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+      const int n = ns + 16 * i;
+      if (has_p && n < N) end[(long)n * P + p] = S[i];
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < OWN; ++i) {
     const int n = ns + 16 * i;
@@ -185,6 +203,118 @@ state_space_scan_kernel(const float* __restrict__ u, const float* __restrict__ t
       kept[(long)i * channels + c] = at < taps - 1 ? kept_from[(long)at * channels + c]
                                                    : conv_in[(long)(first + at - (taps - 1)) * conv_in_stride + c];
     }
+}
+
+// Long stretches of tokens in segments.  The scan above then runs every segment of a request side by side:
+// the first from the request's state, the others from zero, each leaving its end state E_k in `ends` and
+// the running product of its tokens' a in `cum`.  Two more launches make the rest:
+//   the fold, per (request, head, eight value dims), over the request's segments in order: the state a
+//   segment starts from is I_1 = E_0, I_(k+1) = D_k I_k + E_k (D_k: the segment's whole product), left in
+//   `ends` in E_k's place; the last one is the request's new state (and the block (head 0, dims 0) brings
+//   the convolution's kept inputs up to date);
+//   the carry, per (segment but the first, head, eight value dims): y_t += cum_t (I_k^T C_t), what the
+//   state the segment did not start from adds to its outputs; tokens are independent here.
+// The sums of a token then differ in order from the walk of one chain, by rounding, and which tokens share a
+// segment goes by how the request was cut into steps.
+// spans5 [n][5] = (slot, first token, tokens, first segment, segments).
+#define SS_CARRY 32        // tokens of a segment a block of the carry takes
+template <int OWN>
+__global__ void __launch_bounds__(SS_THREADS)
+state_space_fold_kernel(float* __restrict__ ends, const float* __restrict__ cum, const int32_t* __restrict__ spans5,
+                        const int32_t* __restrict__ segs, float* __restrict__ state, long state_stride, long copy_elems,
+                        long tail_at, const int32_t* __restrict__ positions, const float* __restrict__ conv_in,
+                        long conv_in_stride, int heads, int P, int N, int channels, int taps) {
+  const int slot = spans5[5 * blockIdx.x], first = spans5[5 * blockIdx.x + 1], count = spans5[5 * blockIdx.x + 2];
+  const int seg0 = spans5[5 * blockIdx.x + 3], n_segs = spans5[5 * blockIdx.x + 4];
+  const int h = blockIdx.y;
+  const int ns = threadIdx.x & 15, p = blockIdx.z * (SS_THREADS / 16) + (threadIdx.x >> 4);
+  const bool has_p = p < P;
+  const int start = positions[first];
+  const float* from = state + (long)slot * state_stride + (long)((start + 1) & 1) * copy_elems;
+  float* to = state + (long)slot * state_stride + (long)((start + count - 1) & 1) * copy_elems;
+  float I[OWN];
+#pragma unroll
+  for (int i = 0; i < OWN; ++i) {
+    const int n = ns + 16 * i;
+    I[i] = has_p && n < N ? ends[((long)seg0 * heads + h) * N * P + (long)n * P + p] : 0.0f;
+  }
+  for (int k = 1; k < n_segs; ++k) {
+    const int seg = seg0 + k;
+    const int seg_last = segs[4 * seg + 1] + segs[4 * seg + 2] - 1;
+    const float D = cum[(long)seg_last * heads + h];
+    float* E = ends + ((long)seg * heads + h) * N * P;
+#pragma unroll
+    for (int i = 0; i < OWN; ++i) {
+      const int n = ns + 16 * i;
+      if (has_p && n < N) {
+        const float e = E[(long)n * P + p];
+        E[(long)n * P + p] = I[i];
+        I[i] = fmaf(D, I[i], e);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < OWN; ++i) {
+    const int n = ns + 16 * i;
+    if (has_p && n < N) to[(long)h * N * P + (long)n * P + p] = I[i];
+  }
+  if (blockIdx.y != 0 || blockIdx.z != 0) return;
+  float* kept = to + tail_at;
+  const float* kept_from = from + tail_at;
+  for (int c = threadIdx.x; c < channels; c += blockDim.x)
+    for (int i = 0; i < taps - 1; ++i) {
+      const int at = i + count;
+      kept[(long)i * channels + c] = at < taps - 1 ? kept_from[(long)at * channels + c]
+                                                   : conv_in[(long)(first + at - (taps - 1)) * conv_in_stride + c];
+    }
+}
+
+template <int OWN>
+__global__ void __launch_bounds__(SS_THREADS)
+state_space_carry_kernel(const float* __restrict__ u, const float* __restrict__ ends, const float* __restrict__ cum,
+                         const int32_t* __restrict__ segs, float* __restrict__ y, int heads, int groups, int P, int N,
+                         int channels, int pieces) {
+  // blockIdx.x: (segment, piece of SS_CARRY tokens of it); tokens are independent here
+  const int seg = blockIdx.x / pieces, piece = blockIdx.x % pieces;
+  if (segs[4 * seg + 3] != 0) return;                 // a request's first segment started from its state
+  const int seg_first = segs[4 * seg + 1], seg_count = segs[4 * seg + 2];
+  if (piece * SS_CARRY >= seg_count) return;
+  const int first = seg_first + piece * SS_CARRY, count = min(SS_CARRY, seg_count - piece * SS_CARRY);
+  const int h = blockIdx.y, g = h / (heads / groups);
+  const int ns = threadIdx.x & 15, p = blockIdx.z * (SS_THREADS / 16) + (threadIdx.x >> 4);
+  const bool has_p = p < P;
+  const int inner = heads * P;
+  const float* carried = ends + ((long)seg * heads + h) * N * P;
+  float I[OWN];
+  int n_of[OWN];
+#pragma unroll
+  for (int i = 0; i < OWN; ++i) {
+    const int n = ns + 16 * i;
+    I[i] = has_p && n < N ? carried[(long)n * P + p] : 0.0f;
+    n_of[i] = min(n, N - 1);
+  }
+  const long c_col = inner + (long)groups * N + (long)g * N;
+  const long out_col = (long)h * P + (has_p ? p : 0);
+  for (int t0 = first; t0 < first + count; t0 += SS_AHEAD) {
+    float C[SS_AHEAD][OWN], c[SS_AHEAD], was[SS_AHEAD];
+#pragma unroll
+    for (int k = 0; k < SS_AHEAD; ++k) {
+      const int t = min(t0 + k, first + count - 1);
+      const float* row = u + (long)t * channels + c_col;
+#pragma unroll
+      for (int i = 0; i < OWN; ++i) C[k][i] = row[n_of[i]];
+      c[k] = cum[(long)t * heads + h];
+      was[k] = y[(long)t * inner + out_col];
+    }
+#pragma unroll
+    for (int k = 0; k < SS_AHEAD; ++k) {
+      float part = 0.0f;
+#pragma unroll
+      for (int i = 0; i < OWN; ++i) part = fmaf(I[i], C[k][i], part);
+      part = ss_row_sum(part);
+      if (t0 + k < first + count && ns == 0 && has_p) y[(long)(t0 + k) * inner + out_col] = fmaf(c[k], part, was[k]);
+    }
+  }
 }
 
 // out[t, part] = ((v / sqrt(mean(v^2) + eps)) gain) with v = y[t, part] silu(z[t, part]): the gate first,
@@ -250,7 +380,8 @@ extern "C" int axk_state_conv(const float* x, long x_stride, const void* w, cons
 extern "C" int axk_state_space_scan(const float* u, const float* terms, const void* d_skip, int d_is_f32, float* state,
                                     long state_stride, long copy_elems, long tail_at, const int32_t* spans, int n_spans,
                                     const int32_t* positions, const int32_t* seq_rows, const float* conv_in, long conv_in_stride,
-                                    float* y, int heads, int groups, int vdim, int n_state, int taps, void* stream) {
+                                    float* y, int heads, int groups, int vdim, int n_state, int taps, const int32_t* segs,
+                                    int n_segs, int longest_seg, const int32_t* spans5, float* ends, float* cum, void* stream) {
   AXK_REQUIRE(n_spans >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && vdim > 0 && n_state > 0 && taps >= 1,
               "state_space_scan: bad sizes spans=%d heads=%d groups=%d vdim=%d state=%d taps=%d", n_spans, heads, groups, vdim,
               n_state, taps);
@@ -263,14 +394,26 @@ extern "C" int axk_state_space_scan(const float* u, const float* terms, const vo
   AXK_REQUIRE((spans != nullptr || seq_rows != nullptr) && positions != nullptr, "state_space_scan: neither spans nor slots, or no positions");
   AXK_REQUIRE(n_spans <= 65535 * 32 && heads <= 65535 && ceil_div(vdim, SS_THREADS / 16) <= 65535, "state_space_scan: %d requests of %d heads", n_spans, heads);
   if (n_spans == 0) return 0;
-  dim3 grid(n_spans, heads, ceil_div(vdim, SS_THREADS / 16));
+  AXK_REQUIRE(segs == nullptr || (n_segs >= n_spans && spans5 != nullptr && ends != nullptr && cum != nullptr && spans != nullptr),
+              "state_space_scan: %d segments of %d requests come with the requests' list, a workspace and the running products",
+              n_segs, n_spans);
+  dim3 grid(segs ? n_segs : n_spans, heads, ceil_div(vdim, SS_THREADS / 16));
+  dim3 grid_fold(n_spans, heads, ceil_div(vdim, SS_THREADS / 16));
+  AXK_REQUIRE(segs == nullptr || longest_seg > 0, "state_space_scan: segments of at most %d tokens", longest_seg);
+  const int pieces = segs ? ceil_div(longest_seg, SS_CARRY) : 1;
+  dim3 grid_carry((unsigned)((long)(segs ? n_segs : 1) * pieces), heads, ceil_div(vdim, SS_THREADS / 16));
   hipStream_t s = (hipStream_t)stream;
 #define SS_ARGS u, terms, d_skip, d_is_f32, state, state_stride, copy_elems, tail_at, spans, positions, seq_rows, conv_in, conv_in_stride, y, \
-                heads, groups, vdim, n_state, channels, taps
+                heads, groups, vdim, n_state, channels, taps, segs, ends, cum
 #define SS_LAUNCH(OWN)                                                                              \
   {                                                                                                 \
     if (n_state == 16 * OWN) state_space_scan_kernel<OWN, true><<<grid, SS_THREADS, 0, s>>>(SS_ARGS); \
     else state_space_scan_kernel<OWN, false><<<grid, SS_THREADS, 0, s>>>(SS_ARGS);                  \
+    if (segs) {                                                                                     \
+      state_space_fold_kernel<OWN><<<grid_fold, SS_THREADS, 0, s>>>(ends, cum, spans5, segs, state, state_stride, copy_elems, tail_at, \
+                                                                    positions, conv_in, conv_in_stride, heads, vdim, n_state, channels, taps); \
+      state_space_carry_kernel<OWN><<<grid_carry, SS_THREADS, 0, s>>>(u, ends, cum, segs, y, heads, groups, vdim, n_state, channels, pieces); \
+    }                                                                                               \
   }
   if (n_state <= 16) SS_LAUNCH(1)
   else if (n_state <= 32) SS_LAUNCH(2)

@@ -95,7 +95,8 @@ _SIGNATURES = {
     "axk_state_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p,
                        c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "axk_state_space_scan": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_long, c_long, c_long, c_void_p, c_int, c_void_p,
-                             c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                             c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p,
+                             c_void_p, c_void_p, c_void_p],
     "axk_gated_group_norm": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int, c_void_p, c_int,
                            c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
@@ -989,11 +990,14 @@ class Kernels:
         return u
 
     def state_space_scan(self, u, terms, d_skip, state, copy_elems: int, tail_at: int, spans, positions, seq_rows, conv_in, y,
-                         heads: int, groups: int, vdim: int, n_state: int, taps: int) -> torch.Tensor:
+                         heads: int, groups: int, vdim: int, n_state: int, taps: int, segments=None) -> torch.Tensor:
         """The state-space recurrence over each request's tokens (see csrc/state_space.hip): u [T, heads vdim +
         2 groups n_state] and terms [T, heads, 2] float32; spans int32 [n, 3] = (slot, first token, tokens) or None
         (each token a request of its own in slot seq_rows[t]); conv_in: the convolution's inputs (float32, rows may
-        be strided), kept for the next step; y [T, heads vdim] float32."""
+        be strided), kept for the next step; y [T, heads vdim] float32.  `segments` = (segs int32 [n, 4]: slot,
+        first token, tokens, whether the request's first; spans5 int32 [requests, 5]: slot, first token, tokens,
+        first segment, segments; the longest segment's tokens): long stretches run in segments side by side and are folded (sums in another
+        order, by rounding)."""
         for t, what in ((u, "scan u"), (terms, "scan terms"), (state, "scan state"), (y, "scan y")):
             self._f32(t, what)
         self._f32_rows(conv_in, "scan conv_in")
@@ -1008,10 +1012,20 @@ class Kernels:
             n = spans.shape[0]
         else:
             n = T
+        segs = spans5 = ends = cum = None
+        n_segs = longest = 0
+        if segments is not None:
+            segs, spans5, longest = segments
+            self._i32(segs, "scan segments"); self._i32(spans5, "scan requests")
+            n_segs = segs.shape[0]
+            if spans is None or segs.dim() != 2 or segs.shape[1] != 4 or spans5.shape != (n, 5):
+                raise KernelError(f"state_space_scan: segments {tuple(segs.shape)} of requests {tuple(spans5.shape)} for {n} requests")
+            ends = torch.empty((n_segs, heads, n_state, vdim), dtype=torch.float32, device=u.device)
+            cum = torch.empty((T, heads), dtype=torch.float32, device=u.device)
         self._check(self.lib.axk_state_space_scan(
             _ptr(u), _ptr(terms), _ptr(d_skip), self._vec_flag(d_skip, "D"), _ptr(state), state.stride(0), int(copy_elems),
             int(tail_at), _ptr(spans), n, _ptr(positions), _ptr(seq_rows), _ptr(conv_in), conv_in.stride(0), _ptr(y), heads,
-            groups, vdim, n_state, taps, _stream()))
+            groups, vdim, n_state, taps, _ptr(segs), n_segs, int(longest), _ptr(spans5), _ptr(ends), _ptr(cum), _stream()))
         return y
 
     def gated_group_norm(self, y, z, gain, eps: float, out, parts: int) -> torch.Tensor:

@@ -12,7 +12,10 @@ and the output is Wo (rms in `norm_groups` equal parts of (y silu(z)) * gain).  
 convolution's result, dt, the decays, the state and the norm are 32-bit; a request's state row holds S
 and the convolution's last conv - 1 inputs, twice: the state behind position p in copy p & 1, so that a
 decoding step reads one copy and writes the other and may be run again (the engine runs a step once
-before it captures it into a graph) with the same result.
+before it captures it into a graph) with the same result.  Where the walk of one chain a request would leave most of the chip idle, a long
+stretch of a request's tokens in one step runs in segments side by side, each from a zero state but the first,
+whose end states are then folded in order and whose carried-in states' share is added to the outputs: the same
+sums in another order.
 
 Parameters: `hidden_size`, `heads`, `vdim`, `state`, `groups`, `conv`, `norm_groups`, `eps`, `names` (the
 tensors' names under the prefix: scope "mix.", in, conv, dt_bias, A_log, D, norm, o; the convolution's
@@ -28,6 +31,40 @@ from ..config.base import ConfigError
 from ..kernels import MODE_ADD_F32, MODE_STORE_F32
 from .base import CacheBinding, Mixer, StateSpec, TensorDecl, register_mixer
 from .recurrent import step_spans
+
+SEGMENT = 128           # the fewest tokens a segment of a long stretch (a request's tokens of one step) holds
+TARGET_BLOCKS = 2048    # blocks the segmented scan launches: eight a compute unit
+FEW_BLOCKS = 256        # a walk of one chain a request that launches more blocks than this is left as it is
+
+
+def step_segments(ctx, blocks_a_stretch: int):
+    """The stretches of a step cut into segments, for the scan that runs a long stretch's segments side by side:
+    (segs int32 [n, 4] = (slot, first token, tokens, whether the request's first), spans5 int32 [requests, 5] =
+    (slot, first token, tokens, first segment, segments), the longest segment's tokens) on the device, made once a step and scan shape.  A walk
+    of one chain a stretch launches `blocks_a_stretch` blocks a stretch; stretches are cut into as many equal
+    segments (of SEGMENT tokens at least) as brings the launch to TARGET_BLOCKS.  None where that is one segment
+    a stretch, where the walk of one chain a request fills the chip by itself (measured: 512 blocks walk 2,048
+    tokens in 556 us, in four segments each they take 611 with the two further launches; 256 blocks take 533 us
+    and, in eight segments, 337), and in steps of single tokens: one walk a request then, whose sums do not depend
+    on the cuts."""
+    if ctx.decode_only or blocks_a_stretch * len(ctx.spans) > FEW_BLOCKS:
+        return None
+    most = TARGET_BLOCKS // max(1, blocks_a_stretch * len(ctx.spans))
+    if most < 2 or all(s.q_len < 2 * SEGMENT for s in ctx.spans):
+        return None
+    key = ("state_space_segments", most)
+    made = ctx.shared.get(key)
+    if made is None:
+        segs, spans5 = [], []
+        for s in ctx.spans:
+            n = max(1, min(most, s.q_len // SEGMENT))
+            size = -(-s.q_len // n)
+            spans5.append([s.slot, s.q_start, s.q_len, len(segs), -(-s.q_len // size)])
+            for at in range(0, s.q_len, size):
+                segs.append([s.slot, s.q_start + at, min(size, s.q_len - at), 1 if at == 0 else 0])
+        made = ctx.shared[key] = (torch.tensor(segs, dtype=torch.int32).to(ctx.rt.device),
+                                  torch.tensor(spans5, dtype=torch.int32).to(ctx.rt.device), max(r[2] for r in segs))
+    return made
 
 
 class SelectiveStateSpace(Mixer):
@@ -91,7 +128,8 @@ class SelectiveStateSpace(Mixer):
                      silu=True, raw=raw, dt_bias=self.dt_bias, a_log=self.a_log, terms=terms)
         y = ctx.ws.take((T, self.inner), f32)
         k.state_space_scan(u, terms, self.d_skip, state, self.copy_elems, self.tail_at, step_spans(ctx), ctx.positions,
-                           ctx.seq_rows, xbc, y, self.heads, self.groups, self.vdim, self.n_state, self.taps)
+                           ctx.seq_rows, xbc, y, self.heads, self.groups, self.vdim, self.n_state, self.taps,
+                           segments=step_segments(ctx, self.heads * -(-self.vdim // 8)))
         normed = ctx.ws.take((T, self.inner), ctx.rt.dtype)
         k.gated_group_norm(y, z, self.gain, self.eps, normed, self.norm_groups)
         k.gemm(normed, self.w_o, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
