@@ -211,6 +211,33 @@ def test_unequal_requests_side_by_side_with_pages_and_slots_used_again(folders, 
         assert float((alone[2] - got[2]).abs().max()) <= 2 * tolerance(dtype, plain_logits(name, seqs[2]))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_long_stretches_run_the_scan_in_segments(folders, plain_logits, name, dtype):
+    """Hundreds of tokens of a request in one step: the scan cuts the stretch into segments that run side by side,
+    folds their end states and adds the carried-in states' share; the state it leaves is what later portions and
+    decoded tokens go on from.  Beside a short request in the same step, whose stretch is one segment."""
+    n = 420
+    long, short = sequences(name, [n, 9], seed=5)
+    page = MODELS[name]["page"]
+    eng = engine_for(folders(name), dtype, page, -(-n // page) + 4, max_seqs=2, max_seq_len=448, max_batch_tokens=512)
+    seen = []
+    inner = eng.rt.k.state_space_scan
+
+    def logged(*a, segments=None, **kw):
+        seen.append(None if segments is None else segments[0].shape[0])
+        return inner(*a, segments=segments, **kw)
+    eng.rt.k.state_space_scan = logged
+    try:
+        got, chose = run_schedule(eng, name, {"a": long, "b": short}, [[("a", 300), ("b", 4)], [("a", 1), ("b", 5)], [("a", 2)], [("a", 117)]])
+    finally:
+        del eng.rt.k.state_space_scan
+    assert any(k is not None and k > 2 for k in seen) and any(k is None for k in seen)
+    assert_close(got["a"], plain_logits(name, long, dtype, chose["a"]), dtype, "the long request")
+    assert_close(got["b"], plain_logits(name, short, dtype, chose["b"]), dtype, "the short request beside it")
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("name", ["A", "D"])
 def test_long_decoding_across_many_pages(folders, plain_logits, name):
     n = 250
